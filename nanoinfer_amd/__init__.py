@@ -9,8 +9,10 @@ from . import registry
 from .parts import standard as _standard_parts   # registers the parts
 from .parts import hybrid as _hybrid_parts       # registers the parallel block, the mixers with a memory, routed experts
 from .parts import stateful as _stateful_parts   # registers mixers with a state of fixed size, the windowed attention, the pair-hash embedding
+from .parts import gated as _gated_parts         # registers the sandwich block, attention over keys or a latent, the gated matrix memory, the depth average
 from .architectures import llama as _llama       # registers LlamaForCausalLM
 from .architectures import zekalorn as _zekalorn  # registers Zekalorn
 from .architectures import fusavik as _fusavik    # registers Fusavik
+from .architectures import ruludra as _ruludra    # registers Ruludra
 
 __version__ = "0.1.0"

@@ -82,6 +82,9 @@ class ModelSpec:
     ignorable_suffixes: tuple = ()
     # what entries of the order with ``enter`` add to the stream (None: no entry has one)
     pass_input: Optional[PartSpec] = None
+    # a part of family ``stream_mix``: after every entry of the order the stream that goes on is a mix of the
+    # embedding's output and of every entry's own result so far (None: an entry's result goes on as it is)
+    stream_mix: Optional[PartSpec] = None
 
     def num_caches(self) -> int:
         return 1 + max((r.cache for r in self.order), default=-1)

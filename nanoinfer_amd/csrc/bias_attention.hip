@@ -76,7 +76,8 @@ __global__ void kv_store_kernel(const T* __restrict__ qkv, int row_stride, int k
 //   (all heads at once; a null weight: no norm), the rotation turns channel c < rot/2 of every head together with
 //   channel c + rot/2 by the angle position * freq[c], cos and sin times `amplitude` (a null freq: no rotation);
 //   the channels from `rot` on pass as they are.
-// proj float32 [T, row_stride] holds q [H * dk] | k [G * dk] | v [G * dv]; q goes to q_out [T, H * dk] in the compute
+// proj float32 [T, row_stride] holds q [H * dk] | k [G * dk] | v [G * dv] (`v_from_k`: no v; the values are the keys as
+// projected, before their norm, and dv = dk); q goes to q_out [T, H * dk] in the compute
 // type, k and v into their page slots.  A token is taken by gridDim.y workgroups, each with its share of the elements
 // (and the sums of squares over the whole projections, which every one of them works out): one for steps of many
 // tokens; a step of few tokens, where one workgroup a token would walk its row alone, spreads the row.
@@ -87,7 +88,7 @@ __global__ void __launch_bounds__(256)
 qk_norm_rope_store_kernel(const float* __restrict__ proj, int row_stride, const int32_t* __restrict__ positions,
                           const int32_t* __restrict__ slot_mapping, const float* __restrict__ wq, const float* __restrict__ wk,
                           float eps, const float* __restrict__ freq, int rot, float amplitude, T* __restrict__ q_out,
-                          T* __restrict__ kpool, T* __restrict__ vpool, int H, int G, int dk, int dv, int page_size) {
+                          T* __restrict__ kpool, T* __restrict__ vpool, int H, int G, int dk, int dv, int page_size, bool v_from_k) {
     __shared__ float scratch[8];
     __shared__ float cos_of[ROT_PAIRS], sin_of[ROT_PAIRS];     // the token's angles, worked out once for all heads
     const int t = blockIdx.x, tid = threadIdx.x;
@@ -142,7 +143,7 @@ qk_norm_rope_store_kernel(const float* __restrict__ proj, int row_stride, const 
         }
     }
     if (slot >= 0) {
-        const float* vsrc = row + nq + nk;
+        const float* vsrc = v_from_k ? row + nq : row + nq + nk;      // the values may be the keys as projected, before their norm
         const int vper = (G * dv + slices - 1) / slices;
         for (int i = slice * vper + tid; i < min(G * dv, (slice + 1) * vper); i += blockDim.x) {
             const int g = i / dv, c = i % dv;
@@ -154,20 +155,21 @@ qk_norm_rope_store_kernel(const float* __restrict__ proj, int row_stride, const 
 NI_EXPORT int ni_qk_norm_rope_store(const void* proj, int row_stride, const void* positions, const void* slot_mapping,
                                     const void* wq, const void* wk, float eps, const void* freq, int rot, float amplitude,
                                     void* q_out, void* kpool, void* vpool, int T, int H, int G, int dk, int dv, int page_size,
-                                    int dtype, hipStream_t stream) {
+                                    int v_from_k, int dtype, hipStream_t stream) {
     if (T <= 0) return 0;
-    if (rot < 0 || rot > dk || rot % 2 || rot > 2 * ROT_PAIRS || row_stride < H * dk + G * dk + G * dv) return -1;
+    if (rot < 0 || rot > dk || rot % 2 || rot > 2 * ROT_PAIRS || row_stride < H * dk + G * dk + (v_from_k ? 0 : G * dv)) return -1;
+    if (v_from_k && dv != dk) return -1;
     // few tokens: a row's elements over several workgroups, one pass of 256 threads each
     const int slices = T >= 64 ? 1 : std::max(1, std::min(16, ((H + G) * dk + 255) / 256));
     const dim3 grid(T, slices);
     if (dtype == 0)
         qk_norm_rope_store_kernel<float><<<grid, 256, 0, stream>>>((const float*)proj, row_stride, (const int32_t*)positions,
             (const int32_t*)slot_mapping, (const float*)wq, (const float*)wk, eps, (const float*)freq, rot, amplitude,
-            (float*)q_out, (float*)kpool, (float*)vpool, H, G, dk, dv, page_size);
+            (float*)q_out, (float*)kpool, (float*)vpool, H, G, dk, dv, page_size, v_from_k != 0);
     else
         qk_norm_rope_store_kernel<bf16_t><<<grid, 256, 0, stream>>>((const float*)proj, row_stride, (const int32_t*)positions,
             (const int32_t*)slot_mapping, (const float*)wq, (const float*)wk, eps, (const float*)freq, rot, amplitude,
-            (bf16_t*)q_out, (bf16_t*)kpool, (bf16_t*)vpool, H, G, dk, dv, page_size);
+            (bf16_t*)q_out, (bf16_t*)kpool, (bf16_t*)vpool, H, G, dk, dv, page_size, v_from_k != 0);
     return NI_LAUNCH_RESULT();
 }
 

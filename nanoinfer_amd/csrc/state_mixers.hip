@@ -569,3 +569,297 @@ NI_EXPORT int ni_selective_scan(const void* dt_pre, const void* dt_bias, const v
                             inner, N, parts, max_q_len, runs, y_local, dt_sum, RUN, stream);
     return NI_LAUNCH_RESULT();
 }
+
+// ---------------------------------------------------------------- matrix memory with exponential gates
+// Per head, with a memory S [dk, dv], a normaliser n [dk] and a running maximum m of the gates' logarithms, all float32:
+//   li = cap tanh((zi + bi) / cap),  lf = logsigmoid(cap tanh((zf + bf) / cap))
+//   m' = max(lf + m, li);  S <- exp(lf + m - m') S + exp(li - m') k v^T;  n likewise with k alone;  m <- m'
+//   o = S^T q / (max(|n . q|, exp(-m)) + 1e-6)
+// The normaliser is kept as one more value channel whose value is always 1: a slot's state is [H][dv + 1][dkp]
+// (a column of key channels lies together, dkp = parts * 8 >= dk, padding zero) and then m [H].  proj float32
+// [T, stride] holds q, k [H dk each], v [H dv] and the gates' pre-activations zi [H], zf [H] at given columns.  The
+// recurrence kernels leave the raw read-outs [T, H (dv + 1)] (the last of a head is n . q) and m [T, H];
+// memory_norm_kernel divides, norms every head, gates, and keeps the last m of every sequence in the state.
+struct MemoryOperands {
+    float q[DKPT], k[DKPT], v, li, lf;
+};
+
+__device__ __forceinline__ float log_sigmoid_f(float x) { return fminf(x, 0.f) - log1pf(expf(-fabsf(x))); }
+
+__device__ __forceinline__ void memory_load(MemoryOperands& o, const float* __restrict__ row, int q_off, int k_off, int v_off,
+                                            int zi_off, int zf_off, float bi, float bf, float cap, float q_scale, int ch, int dk,
+                                            bool whole, bool ones) {
+    if (whole) {
+        const float4 a = *reinterpret_cast<const float4*>(row + q_off + ch), b = *reinterpret_cast<const float4*>(row + q_off + ch + 4);
+        const float4 c = *reinterpret_cast<const float4*>(row + k_off + ch), d = *reinterpret_cast<const float4*>(row + k_off + ch + 4);
+        o.q[0] = a.x; o.q[1] = a.y; o.q[2] = a.z; o.q[3] = a.w; o.q[4] = b.x; o.q[5] = b.y; o.q[6] = b.z; o.q[7] = b.w;
+        o.k[0] = c.x; o.k[1] = c.y; o.k[2] = c.z; o.k[3] = c.w; o.k[4] = d.x; o.k[5] = d.y; o.k[6] = d.z; o.k[7] = d.w;
+    } else {
+#pragma unroll
+        for (int i = 0; i < DKPT; ++i) {
+            const bool in = ch + i < dk;
+            o.q[i] = in ? row[q_off + ch + i] : 0.f;
+            o.k[i] = in ? row[k_off + ch + i] : 0.f;
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < DKPT; ++i) o.q[i] *= q_scale;
+    o.v = ones ? 1.f : row[v_off];
+    o.li = cap * tanhf((row[zi_off] + bi) / cap);
+    o.lf = log_sigmoid_f(cap * tanhf((row[zf_off] + bf) / cap));
+}
+
+// Token by token from the state (LOCAL false), or a run of RUN tokens from an empty memory whose maximum starts at
+// minus infinity (LOCAL true; the runs' layout is decay_attention_kernel's).  A LOCAL run also leaves, per token, the
+// sum of lf since the run's start (`since`), and per run and head (its maximum at the end, that sum at the end).
+template <bool LOCAL>
+__global__ void __launch_bounds__(256)
+memory_steps_kernel(const float* __restrict__ proj, int stride, int q_col, int k_col, int v_col, int z_col,
+                    const float* __restrict__ gate_bias, float cap, float q_scale, const float* __restrict__ state,
+                    float* __restrict__ state_out, size_t state_stride, const int32_t* __restrict__ q_start,
+                    const int32_t* __restrict__ q_len, const int32_t* __restrict__ state_slot, float* __restrict__ out,
+                    float* __restrict__ m_out, float* __restrict__ since, float* __restrict__ run_ends, int H, int dk, int dv,
+                    int parts, float* __restrict__ runs, int xblocks, int RUN) {
+    const int b = blockIdx.z, h = blockIdx.y;
+    const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
+    const int cols = WAVE / parts;
+    const int part = lane % parts;
+    const int run = LOCAL ? blockIdx.x / xblocks : 0, xb = LOCAL ? blockIdx.x % xblocks : blockIdx.x;
+    const int c = (xb * (blockDim.x / WAVE) + wave) * cols + lane / parts;
+    const int first = run * RUN;
+    const int n = LOCAL ? min(q_len[b] - first, RUN) : q_len[b];
+    const int dvn = dv + 1;
+    if (c >= dvn || n <= 0) return;               // whole groups of `parts` lanes leave together
+    const int dkp = parts * DKPT, ch = part * DKPT;
+    const size_t heads_floats = static_cast<size_t>(H) * dvn * dkp;
+    const size_t run_index = LOCAL ? static_cast<size_t>(q_start[b] / RUN + b + run) : 0;
+    const size_t at = (static_cast<size_t>(h) * dvn + c) * dkp + ch;
+    float S[DKPT];
+    float m;
+    if (LOCAL) {
+#pragma unroll
+        for (int i = 0; i < DKPT; ++i) S[i] = 0.f;
+        m = -INFINITY;
+    } else {
+        const float* srow = state + static_cast<size_t>(state_slot[b]) * state_stride;
+        const float4 a = *reinterpret_cast<const float4*>(srow + at), d = *reinterpret_cast<const float4*>(srow + at + 4);
+        S[0] = a.x; S[1] = a.y; S[2] = a.z; S[3] = a.w; S[4] = d.x; S[5] = d.y; S[6] = d.z; S[7] = d.w;
+        m = srow[heads_floats + h];
+    }
+    const float bi = gate_bias[h], bf = gate_bias[H + h];
+    const int q_off = q_col + h * dk, k_off = k_col + h * dk, v_off = v_col + h * dv + c, zi_off = z_col + h, zf_off = z_col + H + h;
+    const bool whole = dk % DKPT == 0 && ch + DKPT <= dk && stride % 4 == 0 && q_col % 4 == 0 && k_col % 4 == 0;
+    const bool idle = ch >= dk;                   // a lane that holds padding only
+    const bool ones = c == dv;                    // the normaliser's column
+    const bool scribe = xb == 0 && wave == 0 && lane == 0;     // the one thread of (sequence, head, run) that writes the scalars
+    const int t0 = q_start[b] + first;
+    float passed = 0.f;                           // sum of lf since the run's start
+    MemoryOperands cur, nxt;
+    memory_load(cur, proj + static_cast<size_t>(t0) * stride, q_off, k_off, v_off, zi_off, zf_off, bi, bf, cap, q_scale, ch, dk, whole && !idle, ones);
+    for (int r = 0; r < n; ++r) {
+        if (r + 1 < n)
+            memory_load(nxt, proj + static_cast<size_t>(t0 + r + 1) * stride, q_off, k_off, v_off, zi_off, zf_off, bi, bf, cap, q_scale,
+                        ch, dk, whole && !idle, ones);
+        const float m_new = fmaxf(cur.lf + m, cur.li);
+        const float keep = expf(cur.lf + m - m_new), take = expf(cur.li - m_new) * cur.v;
+        float sum = 0.f;
+        if (!idle) {
+#pragma unroll
+            for (int i = 0; i < DKPT; ++i) {
+                S[i] = keep * S[i] + take * cur.k[i];
+                sum += S[i] * cur.q[i];
+            }
+        }
+        m = m_new;
+        passed += cur.lf;
+        sum = parts_sum(sum, parts);
+        if (part == 0) out[static_cast<size_t>(t0 + r) * (H * dvn) + h * dvn + c] = sum;
+        if (scribe) {
+            m_out[static_cast<size_t>(t0 + r) * H + h] = m;
+            if (LOCAL) since[static_cast<size_t>(t0 + r) * H + h] = passed;
+        }
+        cur = nxt;
+    }
+    float* dst = LOCAL ? runs + run_index * heads_floats + at : state_out + static_cast<size_t>(state_slot[b]) * state_stride + at;
+    *reinterpret_cast<float4*>(dst) = make_float4(S[0], S[1], S[2], S[3]);
+    *reinterpret_cast<float4*>(dst + 4) = make_float4(S[4], S[5], S[6], S[7]);
+    if (LOCAL && scribe) {
+        run_ends[(run_index * H + h) * 2] = m;
+        run_ends[(run_index * H + h) * 2 + 1] = passed;
+    }
+}
+
+// step 2 of the runs: one thread an element of [H][dv + 1][dkp]; the memory at the start of run r takes the place of
+// what the run adds, and run_starts gets the maximum at the start of every run
+__global__ void memory_chain_kernel(float* __restrict__ runs, const float* __restrict__ run_ends, float* __restrict__ run_starts,
+                                    float* __restrict__ state, size_t state_stride, const int32_t* __restrict__ q_start,
+                                    const int32_t* __restrict__ q_len, const int32_t* __restrict__ state_slot, int per_head, int H,
+                                    int elems, int RUN) {
+    const int e = blockIdx.x * blockDim.x + threadIdx.x, b = blockIdx.y;
+    const int n = q_len[b];
+    if (e >= elems || n <= 0) return;
+    const int h = e / per_head;
+    const size_t base = static_cast<size_t>(q_start[b] / RUN + b);
+    float* srow = state + static_cast<size_t>(state_slot[b]) * state_stride;
+    float S = srow[e];
+    float m = srow[elems + h];
+    const int n_runs = (n + RUN - 1) / RUN;
+    for (int r = 0; r < n_runs; ++r) {
+        float* at = runs + (base + r) * elems + e;
+        const float add = *at;
+        *at = S;
+        if (e % per_head == 0) run_starts[(base + r) * H + h] = m;
+        const float end_max = run_ends[((base + r) * H + h) * 2], passed = run_ends[((base + r) * H + h) * 2 + 1];
+        const float m_new = fmaxf(passed + m, end_max);
+        S = expf(passed + m - m_new) * S + expf(end_max - m_new) * add;
+        m = m_new;
+    }
+    srow[e] = S;          // (the maximum itself is kept by memory_norm_kernel: other threads of this launch still read it)
+}
+
+// step 3 of the runs: what the memory at a run's start gives its tokens, and every token's own maximum
+__global__ void __launch_bounds__(256)
+memory_carry_kernel(const float* __restrict__ proj, int stride, int q_col, float q_scale, const float* __restrict__ runs,
+                    const float* __restrict__ run_starts, const float* __restrict__ local_max, const float* __restrict__ since,
+                    const int32_t* __restrict__ q_start, const int32_t* __restrict__ q_len, float* __restrict__ out,
+                    float* __restrict__ m_out, int H, int dk, int dv, int parts, int xblocks, int RUN) {
+    const int b = blockIdx.z, h = blockIdx.y;
+    const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
+    const int cols = WAVE / parts;
+    const int part = lane % parts;
+    const int run = blockIdx.x / xblocks, xb = blockIdx.x % xblocks;
+    const int c = (xb * (blockDim.x / WAVE) + wave) * cols + lane / parts;
+    const int first = run * RUN;
+    const int n = min(q_len[b] - first, RUN);
+    const int dvn = dv + 1;
+    if (c >= dvn || n <= 0) return;
+    const int dkp = parts * DKPT, ch = part * DKPT;
+    const size_t run_index = static_cast<size_t>(q_start[b] / RUN + b + run);
+    const float* srow = runs + run_index * H * dvn * dkp + (static_cast<size_t>(h) * dvn + c) * dkp + ch;
+    float S[DKPT];
+    {
+        const float4 a = *reinterpret_cast<const float4*>(srow), d = *reinterpret_cast<const float4*>(srow + 4);
+        S[0] = a.x; S[1] = a.y; S[2] = a.z; S[3] = a.w; S[4] = d.x; S[5] = d.y; S[6] = d.z; S[7] = d.w;
+    }
+    const float m0 = run_starts[run_index * H + h];
+    const int q_off = q_col + h * dk + ch;
+    const bool whole = dk % DKPT == 0 && ch + DKPT <= dk && stride % 4 == 0 && q_col % 4 == 0;
+    const bool idle = ch >= dk;
+    const bool scribe = xb == 0 && wave == 0 && lane == 0;
+    const int t0 = q_start[b] + first;
+    for (int r = 0; r < n; ++r) {
+        const float* row = proj + static_cast<size_t>(t0 + r) * stride + q_off;
+        float sum = 0.f;
+        if (!idle) {
+            if (whole) {
+                const float4 a = *reinterpret_cast<const float4*>(row), d = *reinterpret_cast<const float4*>(row + 4);
+                sum = S[0] * a.x + S[1] * a.y + S[2] * a.z + S[3] * a.w + S[4] * d.x + S[5] * d.y + S[6] * d.z + S[7] * d.w;
+            } else {
+#pragma unroll
+                for (int i = 0; i < DKPT; ++i) sum += ch + i < dk ? S[i] * row[i] : 0.f;
+            }
+        }
+        sum = parts_sum(sum, parts) * q_scale;
+        const size_t th = static_cast<size_t>(t0 + r) * H + h;
+        const float own = local_max[th], before = since[th] + m0;
+        const float m = fmaxf(before, own);
+        if (part == 0) {
+            float* o = out + static_cast<size_t>(t0 + r) * (H * dvn) + h * dvn + c;
+            *o = expf(own - m) * *o + expf(before - m) * sum;
+        }
+        if (scribe) m_out[th] = m;
+    }
+}
+
+// y[t, h dv + c] = N_h(o / (max(|n . q|, exp(-m)) + 1e-6)) * w * sigmoid(gate): N_h divides a head's dv numbers by their
+// root mean square.  raw float32 [T, H (dv + 1)], m float32 [T, H]; a workgroup a token, a wavefront a head at a time.
+// The last token of every sequence's portion leaves its m in the state (behind the memories, at `m_off`).
+template <typename T>
+__global__ void __launch_bounds__(256)
+memory_norm_kernel(const float* __restrict__ raw, const float* __restrict__ m_of, const float* __restrict__ gate, int gate_stride,
+                   const float* __restrict__ w, T* __restrict__ y, float* __restrict__ state, size_t state_stride, size_t m_off,
+                   const int32_t* __restrict__ seq_of_token, const int32_t* __restrict__ q_start, const int32_t* __restrict__ q_len,
+                   const int32_t* __restrict__ state_slot, int H, int dv, float eps) {
+    const int t = blockIdx.x;
+    const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE, waves = blockDim.x / WAVE;
+    const int dvn = dv + 1;
+    const int b = seq_of_token[t];
+    const bool last = t == q_start[b] + q_len[b] - 1;
+    for (int h = wave; h < H; h += waves) {
+        const float* row = raw + static_cast<size_t>(t) * H * dvn + static_cast<size_t>(h) * dvn;
+        const float m = m_of[static_cast<size_t>(t) * H + h];
+        const float inv = 1.0f / (fmaxf(fabsf(row[dv]), expf(-m)) + 1e-6f);
+        float ss = 0.f;
+        for (int c = lane; c < dv; c += WAVE) {
+            const float v = row[c] * inv;
+            ss += v * v;
+        }
+        const float r = 1.0f / sqrtf(wave_sum(ss) / static_cast<float>(dv) + eps);
+        const float* g = gate + static_cast<size_t>(t) * gate_stride + h * dv;
+        for (int c = lane; c < dv; c += WAVE)
+            st(y + static_cast<size_t>(t) * H * dv + h * dv + c, (row[c] * inv) * r * w[h * dv + c] * sigmoid_f(g[c]));
+        if (last && lane == 0) state[static_cast<size_t>(state_slot[b]) * state_stride + m_off + h] = m;
+    }
+}
+
+NI_EXPORT int ni_memory_norm(const void* raw, const void* m_of, const void* gate, int gate_stride, const void* w, void* y,
+                             void* state, size_t state_stride, size_t m_off, const void* seq_of_token, const void* q_start,
+                             const void* q_len, const void* state_slot, int T, int H, int dv, float eps, int dtype, hipStream_t stream) {
+    if (T <= 0) return 0;
+    if (gate_stride < H * dv || state_stride < m_off + H) return -1;
+    const int threads = H >= 4 ? 256 : 64 * H;
+    if (dtype == 0)
+        memory_norm_kernel<float><<<T, threads, 0, stream>>>((const float*)raw, (const float*)m_of, (const float*)gate, gate_stride,
+            (const float*)w, (float*)y, (float*)state, state_stride, m_off, (const int32_t*)seq_of_token, (const int32_t*)q_start,
+            (const int32_t*)q_len, (const int32_t*)state_slot, H, dv, eps);
+    else
+        memory_norm_kernel<bf16_t><<<T, threads, 0, stream>>>((const float*)raw, (const float*)m_of, (const float*)gate, gate_stride,
+            (const float*)w, (bf16_t*)y, (float*)state, state_stride, m_off, (const int32_t*)seq_of_token, (const int32_t*)q_start,
+            (const int32_t*)q_len, (const int32_t*)state_slot, H, dv, eps);
+    return NI_LAUNCH_RESULT();
+}
+
+// `scalars` (float32, 3 T H + 3 (T / RUN + B) H; the first T H only without runs): the tokens' local maxima and sums of
+// lf, and the runs' ends and starts.  `runs` (float32, (T / RUN + B) H (dv + 1) dkp, or null) switches the runs on.
+// m_out float32 [T, H]; out float32 [T, H (dv + 1)].
+NI_EXPORT int ni_gated_memory(const void* proj, int stride, int q_col, int k_col, int v_col, int z_col, const void* gate_bias,
+                              float cap, float q_scale, void* state, size_t state_stride, const void* q_start, const void* q_len,
+                              const void* state_slot, void* out, void* m_out, int T, int B, int H, int dk, int dv, int max_q_len,
+                              void* runs, void* scalars, int RUN, hipStream_t stream) {
+    if (T <= 0 || B <= 0) return 0;
+    const int parts = ni_decay_attention_parts(dk);
+    const int dvn = dv + 1;
+    const size_t heads_floats = static_cast<size_t>(H) * dvn * parts * DKPT;
+    if (!parts || state_stride < heads_floats + H || !(cap > 0.f)) return -1;
+    if (stride < q_col + H * dk || stride < k_col + H * dk || stride < v_col + H * dv || stride < z_col + 2 * H) return -1;
+    if (reinterpret_cast<uintptr_t>(state) % 16 || state_stride % 4 || reinterpret_cast<uintptr_t>(proj) % 16) return -1;
+    const int cols = 4 * (WAVE / parts);
+    const int xblocks = (dvn + cols - 1) / cols;
+    if (!runs) {
+        dim3 grid(xblocks, H, B);
+        memory_steps_kernel<false><<<grid, 256, 0, stream>>>((const float*)proj, stride, q_col, k_col, v_col, z_col,
+            (const float*)gate_bias, cap, q_scale, (const float*)state, (float*)state, state_stride, (const int32_t*)q_start,
+            (const int32_t*)q_len, (const int32_t*)state_slot, (float*)out, (float*)m_out, nullptr, nullptr, H, dk, dv, parts, nullptr,
+            xblocks, 0);
+        return NI_LAUNCH_RESULT();
+    }
+    if (max_q_len < 1 || max_q_len > T || RUN < 1 || !scalars || reinterpret_cast<uintptr_t>(runs) % 16) return -1;
+    const size_t max_runs = static_cast<size_t>(T / RUN + B);
+    float* local_max = (float*)scalars;
+    float* since = local_max + static_cast<size_t>(T) * H;
+    float* run_ends = since + static_cast<size_t>(T) * H;
+    float* run_starts = run_ends + max_runs * H * 2;
+    const int n_runs = (max_q_len + RUN - 1) / RUN;
+    dim3 grid(xblocks * n_runs, H, B);
+    memory_steps_kernel<true><<<grid, 256, 0, stream>>>((const float*)proj, stride, q_col, k_col, v_col, z_col,
+        (const float*)gate_bias, cap, q_scale, nullptr, nullptr, 0, (const int32_t*)q_start, (const int32_t*)q_len,
+        (const int32_t*)state_slot, (float*)out, local_max, since, run_ends, H, dk, dv, parts, (float*)runs, xblocks, RUN);
+    const int elems = static_cast<int>(heads_floats);
+    dim3 chain(blocks_of(elems, 256), B);
+    memory_chain_kernel<<<chain, 256, 0, stream>>>((float*)runs, run_ends, run_starts, (float*)state, state_stride, (const int32_t*)q_start,
+                                                   (const int32_t*)q_len, (const int32_t*)state_slot, dvn * parts * DKPT, H, elems, RUN);
+    memory_carry_kernel<<<grid, 256, 0, stream>>>((const float*)proj, stride, q_col, q_scale, (const float*)runs, run_starts, local_max,
+                                                  since, (const int32_t*)q_start, (const int32_t*)q_len, (float*)out, (float*)m_out, H,
+                                                  dk, dv, parts, xblocks, RUN);
+    return NI_LAUNCH_RESULT();
+}

@@ -58,18 +58,21 @@ NI_EXPORT int ni_embed_scaled(const void* ids, const void* positions, const void
 // out[t] = table[ids[t]] * scale + pairs[(prev * mul_prev + ids[t] * mul_cur) mod buckets], prev the token before
 // ids[t] in its sequence; a sequence's first token (position 0) takes row `buckets`.  The token before the first
 // row of a portion is what `last_token[slot]` holds: remember_last_kernel leaves every sequence's last token there
-// after the rows have been read (a launch of its own: the first row of a portion must not see it).
+// after the rows have been read (a launch of its own: the first row of a portion must not see it).  `pairs` may be
+// null (no second table).  With `freq` (float32 [(d + 1) / 2]) a sinusoid of the position is added: column 2i gets
+// sin(position * freq[i]), column 2i + 1 the cosine of the same angle, the angle a float32 product.
 template <typename T>
 __global__ void embed_pair_hash_kernel(const int32_t* __restrict__ ids, const int32_t* __restrict__ positions,
                                        const int32_t* __restrict__ seq_of_token, const int32_t* __restrict__ q_start,
                                        const int32_t* __restrict__ state_slot, const int32_t* __restrict__ last_token,
                                        const T* __restrict__ table, const T* __restrict__ pairs, float* __restrict__ out,
-                                       int d, int vocab, int buckets, long long mul_prev, long long mul_cur, float scale) {
+                                       int d, int vocab, int buckets, long long mul_prev, long long mul_cur, float scale,
+                                       const float* __restrict__ freq) {
     const int t = blockIdx.x;
     const int id = ids[t];
     if (id < 0 || id >= vocab) return;      // unreachable after the host's check
     int row = buckets;
-    if (positions[t] > 0) {
+    if (pairs && positions[t] > 0) {
         const int s = seq_of_token[t];
         const int prev = (t == q_start[s]) ? last_token[state_slot[s]] : ids[t - 1];
         long long r = (static_cast<long long>(prev) * mul_prev + static_cast<long long>(id) * mul_cur) % buckets;
@@ -79,7 +82,16 @@ __global__ void embed_pair_hash_kernel(const int32_t* __restrict__ ids, const in
     const T* erow = table + static_cast<size_t>(id) * d;
     const T* prow = pairs + static_cast<size_t>(row) * d;
     float* o = out + static_cast<size_t>(t) * d;
-    for (int i = threadIdx.x; i < d; i += blockDim.x) o[i] = ld(erow + i) * scale + ld(prow + i);
+    const float pos = static_cast<float>(positions[t]);
+    for (int i = threadIdx.x; i < d; i += blockDim.x) {
+        float v = ld(erow + i) * scale;
+        if (pairs) v += ld(prow + i);
+        if (freq) {
+            const float angle = pos * freq[i / 2];
+            v += (i & 1) ? cosf(angle) : sinf(angle);
+        }
+        o[i] = v;
+    }
 }
 
 __global__ void remember_last_kernel(const int32_t* __restrict__ ids, const int32_t* __restrict__ q_start,
@@ -92,17 +104,17 @@ __global__ void remember_last_kernel(const int32_t* __restrict__ ids, const int3
 NI_EXPORT int ni_embed_pair_hash(const void* ids, const void* positions, const void* seq_of_token, const void* q_start,
                                  const void* q_len, const void* state_slot, void* last_token, const void* table,
                                  const void* pairs, void* out, int T, int B, int d, int vocab, int buckets, long long mul_prev,
-                                 long long mul_cur, float scale, int dtype, hipStream_t stream) {
+                                 long long mul_cur, float scale, const void* freq, int dtype, hipStream_t stream) {
     if (T <= 0 || B <= 0) return 0;
-    if (buckets < 1) return -1;
+    if (pairs && buckets < 1) return -1;
     if (dtype == 0)
         embed_pair_hash_kernel<float><<<T, 256, 0, stream>>>((const int32_t*)ids, (const int32_t*)positions, (const int32_t*)seq_of_token,
             (const int32_t*)q_start, (const int32_t*)state_slot, (const int32_t*)last_token, (const float*)table, (const float*)pairs,
-            (float*)out, d, vocab, buckets, mul_prev, mul_cur, scale);
+            (float*)out, d, vocab, buckets, mul_prev, mul_cur, scale, (const float*)freq);
     else
         embed_pair_hash_kernel<bf16_t><<<T, 256, 0, stream>>>((const int32_t*)ids, (const int32_t*)positions, (const int32_t*)seq_of_token,
             (const int32_t*)q_start, (const int32_t*)state_slot, (const int32_t*)last_token, (const bf16_t*)table, (const bf16_t*)pairs,
-            (float*)out, d, vocab, buckets, mul_prev, mul_cur, scale);
+            (float*)out, d, vocab, buckets, mul_prev, mul_cur, scale, (const float*)freq);
     remember_last_kernel<<<blocks_of(B, 64), 64, 0, stream>>>((const int32_t*)ids, (const int32_t*)q_start, (const int32_t*)q_len,
                                                                (const int32_t*)state_slot, (int32_t*)last_token, B);
     return NI_LAUNCH_RESULT();
@@ -217,6 +229,159 @@ NI_EXPORT int ni_add_rmsnormed(void* h, const void* y, const void* w, int T, int
     if (T <= 0) return 0;
     const int threads = d <= 256 ? 64 : d <= 1024 ? 256 : 512;
     add_rmsnormed_kernel<<<T, threads, 0, stream>>>((float*)h, (const float*)y, (const float*)w, d, eps);
+    return NI_LAUNCH_RESULT();
+}
+
+// ---------------------------------------------------------------- y = x / sqrt(mean(x^2) + eps) * w over columns of wider rows
+// x: n columns of float32 rows of stride `stride` (a product's accumulators); y [T, n] in the type T
+template <typename T>
+__global__ void rmsnorm_cols_kernel(const float* __restrict__ x, int stride, const float* __restrict__ w, T* __restrict__ y,
+                                    int n, float eps) {
+    __shared__ float scratch[16];
+    const float* row = x + static_cast<size_t>(blockIdx.x) * stride;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < n; i += blockDim.x) ss += row[i] * row[i];
+    const float inv = 1.0f / sqrtf(block_sum(ss, scratch) / static_cast<float>(n) + eps);
+    for (int i = threadIdx.x; i < n; i += blockDim.x) st(y + static_cast<size_t>(blockIdx.x) * n + i, (row[i] * inv) * w[i]);
+}
+
+NI_EXPORT int ni_rmsnorm_cols(const void* x, int stride, const void* w, void* y, int T, int n, float eps, int dtype, hipStream_t stream) {
+    if (T <= 0 || n <= 0) return 0;
+    if (stride < n) return -1;
+    const int threads = n <= 256 ? 64 : n <= 1024 ? 256 : 512;
+    if (dtype == 0)
+        rmsnorm_cols_kernel<float><<<T, threads, 0, stream>>>((const float*)x, stride, (const float*)w, (float*)y, n, eps);
+    else
+        rmsnorm_cols_kernel<bf16_t><<<T, threads, 0, stream>>>((const float*)x, stride, (const float*)w, (bf16_t*)y, n, eps);
+    return NI_LAUNCH_RESULT();
+}
+
+// ---------------------------------------------------------------- a weighted sum of earlier states of the stream
+// out[t, :] = sum_j w[j] * hist[j][t, :] for j < n; hist is [n][T][d] float32 (whole streams one after the other)
+__global__ void depth_mix_kernel(const float* __restrict__ hist, const float* __restrict__ w, float* __restrict__ out, int n,
+                                 size_t per, bool pieces) {
+    const size_t i = (static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x) * 4;
+    if (i >= per) return;
+    if (pieces) {           // whole 16-byte pieces: `per` is a multiple of 4 and both buffers are aligned
+        float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+        for (int j = 0; j < n; ++j) {
+            const float4 v = *reinterpret_cast<const float4*>(hist + static_cast<size_t>(j) * per + i);
+            const float wj = w[j];
+            acc.x += wj * v.x; acc.y += wj * v.y; acc.z += wj * v.z; acc.w += wj * v.w;
+        }
+        *reinterpret_cast<float4*>(out + i) = acc;
+    } else {
+        for (size_t e = i; e < per && e < i + 4; ++e) {
+            float acc = 0.f;
+            for (int j = 0; j < n; ++j) acc += w[j] * hist[static_cast<size_t>(j) * per + e];
+            out[e] = acc;
+        }
+    }
+}
+
+NI_EXPORT int ni_depth_mix(const void* hist, const void* w, void* out, int n, int T, int d, hipStream_t stream) {
+    const size_t per = static_cast<size_t>(T) * d;
+    if (per == 0 || n <= 0) return 0;
+    const bool pieces = per % 4 == 0 && reinterpret_cast<uintptr_t>(hist) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0;
+    depth_mix_kernel<<<blocks_of((per + 3) / 4, 256), 256, 0, stream>>>((const float*)hist, (const float*)w, (float*)out, n, per, pieces);
+    return NI_LAUNCH_RESULT();
+}
+
+// ---------------------------------------------------------------- a polynomial of normed powers as activation
+//   y = a N(z) + b N(z^2) + c N(z^3) + e,   N(u) = u / sqrt(mean(u^2) + eps) over the row, powers element by element
+// z float32 [T, n] (a product's accumulators), coef float32 [4] = (a, b, c, e); y in the type T.  A row is taken by
+// gridDim.y workgroups, each with its share of the elements (and the whole row's three sums).
+template <typename T>
+__global__ void __launch_bounds__(256)
+poly_norm_kernel(const float* __restrict__ z, const float* __restrict__ coef, T* __restrict__ y, int n, float eps) {
+    __shared__ float scratch[16];
+    const float* row = z + static_cast<size_t>(blockIdx.x) * n;
+    float s2 = 0.f, s4 = 0.f, s6 = 0.f;
+    for (int i = threadIdx.x; i < n; i += blockDim.x) {
+        const float v = row[i], v2 = v * v;
+        s2 += v2;
+        s4 += v2 * v2;
+        s6 += v2 * v2 * v2;
+    }
+    s2 = block_sum(s2, scratch);
+    s4 = block_sum(s4, scratch);
+    s6 = block_sum(s6, scratch);
+    const float fn = static_cast<float>(n);
+    const float r1 = coef[0] / sqrtf(s2 / fn + eps), r2 = coef[1] / sqrtf(s4 / fn + eps), r3 = coef[2] / sqrtf(s6 / fn + eps);
+    const float e = coef[3];
+    const int per = (n + gridDim.y - 1) / gridDim.y;
+    for (int i = blockIdx.y * per + threadIdx.x; i < min(n, (blockIdx.y + 1) * per); i += blockDim.x) {
+        const float v = row[i];
+        st(y + static_cast<size_t>(blockIdx.x) * n + i, (v * r1 + (v * v) * r2) + ((v * v * v) * r3 + e));
+    }
+}
+
+NI_EXPORT int ni_poly_norm(const void* z, const void* coef, void* y, int T, int n, float eps, int dtype, hipStream_t stream) {
+    if (T <= 0 || n <= 0) return 0;
+    const dim3 grid(T, T >= 64 ? 1 : std::max(1, std::min(16, (n + 1023) / 1024)));
+    if (dtype == 0)
+        poly_norm_kernel<float><<<grid, 256, 0, stream>>>((const float*)z, (const float*)coef, (float*)y, n, eps);
+    else
+        poly_norm_kernel<bf16_t><<<grid, 256, 0, stream>>>((const float*)z, (const float*)coef, (bf16_t*)y, n, eps);
+    return NI_LAUNCH_RESULT();
+}
+
+// ---------------------------------------------------------------- x *= s, element by element (float32)
+__global__ void scale_kernel(float* __restrict__ x, float s, size_t n) {
+    const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i < n) x[i] *= s;
+}
+
+NI_EXPORT int ni_scale(void* x, float s, size_t n, hipStream_t stream) {
+    if (n == 0) return 0;
+    scale_kernel<<<blocks_of(n, 256), 256, 0, stream>>>((float*)x, s, n);
+    return NI_LAUNCH_RESULT();
+}
+
+// ---------------------------------------------------------------- read-outs head by head times a gate
+//   y[t, h * dv + c] = o[h][t][c] * sigmoid(g[t, h * dv + c])      o float32 [H][T][dv], g float32 rows of stride g_stride
+template <typename T>
+__global__ void gate_heads_kernel(const float* __restrict__ o, const float* __restrict__ g, int g_stride, T* __restrict__ y,
+                                  int Tn, int H, int dv, size_t total) {
+    const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    const int c = static_cast<int>(i % dv), h = static_cast<int>((i / dv) % H);
+    const size_t t = i / (static_cast<size_t>(dv) * H);
+    const float gate = 1.0f / (1.0f + expf(-g[t * g_stride + h * dv + c]));
+    st(y + i, o[(static_cast<size_t>(h) * Tn + t) * dv + c] * gate);
+}
+
+NI_EXPORT int ni_gate_heads(const void* o, const void* g, int g_stride, void* y, int T, int H, int dv, int dtype, hipStream_t stream) {
+    const size_t total = static_cast<size_t>(T) * H * dv;
+    if (total == 0) return 0;
+    if (g_stride < H * dv) return -1;
+    if (dtype == 0)
+        gate_heads_kernel<float><<<blocks_of(total, 256), 256, 0, stream>>>((const float*)o, (const float*)g, g_stride, (float*)y, T, H, dv, total);
+    else
+        gate_heads_kernel<bf16_t><<<blocks_of(total, 256), 256, 0, stream>>>((const float*)o, (const float*)g, g_stride, (bf16_t*)y, T, H, dv, total);
+    return NI_LAUNCH_RESULT();
+}
+
+// ---------------------------------------------------------------- rows of heads, token by token, as heads of rows
+//   y[h][t][c] = x[t, h * n + c]      (what a product per head reads: every head's rows together)
+template <typename T>
+__global__ void heads_apart_kernel(const T* __restrict__ x, int x_stride, T* __restrict__ y, int Tn, int H, int n, size_t total) {
+    const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    const int c = static_cast<int>(i % n);
+    const size_t t = (i / n) % Tn;
+    const int h = static_cast<int>(i / (static_cast<size_t>(n) * Tn));
+    y[i] = x[t * x_stride + h * n + c];
+}
+
+NI_EXPORT int ni_heads_apart(const void* x, int x_stride, void* y, int T, int H, int n, int dtype, hipStream_t stream) {
+    const size_t total = static_cast<size_t>(T) * H * n;
+    if (total == 0) return 0;
+    if (x_stride < H * n) return -1;
+    if (dtype == 0)
+        heads_apart_kernel<float><<<blocks_of(total, 256), 256, 0, stream>>>((const float*)x, x_stride, (float*)y, T, H, n, total);
+    else
+        heads_apart_kernel<bf16_t><<<blocks_of(total, 256), 256, 0, stream>>>((const bf16_t*)x, x_stride, (bf16_t*)y, T, H, n, total);
     return NI_LAUNCH_RESULT();
 }
 

@@ -25,6 +25,8 @@ class Model:
         self.blocks = [get_part("block", b.kind)(b, tensors, rt) for b in spec.blocks]
         self.final_norm = build_part("norm", spec.final_norm, tensors, rt)
         self.pass_input = None if spec.pass_input is None else build_part("pass_input", spec.pass_input, tensors, rt)
+        # a mix of all earlier states of the stream that takes an entry's result's place (None: none)
+        self.stream_mix = None if spec.stream_mix is None else build_part("stream_mix", spec.stream_mix, tensors, rt)
         # a function (index of the entry of the order, h) called after every entry with the complete residual
         # stream, for whoever wants to look at a pass layer by layer; None costs nothing
         self.tap = None
@@ -57,7 +59,7 @@ class Model:
 
     def _all_parts(self):
         return [self.embedding, self.final_norm, self.head] + list(self.blocks) + \
-            ([] if self.pass_input is None else [self.pass_input])
+            ([] if self.pass_input is None else [self.pass_input]) + ([] if self.stream_mix is None else [self.stream_mix])
 
     def graph_safe(self) -> bool:
         """Whether a step of this model may be recorded into a HIP graph: every part says of itself
@@ -92,6 +94,15 @@ class Model:
         pending = None
         order = self.spec.order
         T = h.shape[0]
+        history = None
+        if self.stream_mix is not None:
+            # every state of the stream is kept for the step: row 0 the embedding's output, row i + 1 the result of
+            # entry i, which works in place on the row that was filled with what it reads
+            history = torch.empty(len(order) + 1, T, h.shape[1], dtype=torch.float32, device=h.device)
+            history[0].copy_(h)
+            if order:
+                history[1].copy_(h)
+                h = history[1]
         for i, run in enumerate(order):
             cache: LayerCache = layer_cache(run.cache, run.writes_cache)
             block = self.blocks[run.block]
@@ -102,12 +113,19 @@ class Model:
                 h = self.pass_input.forward(h, run.enter) if embedded is None else self.pass_input.forward(h, run.enter, embedded)
             # what the block behind this one would like to find beside the stream (its first norm's input half
             # done by this block's last product), if both blocks know of that
-            wants = getattr(self.blocks[order[i + 1].block], "wants_scaled", None) if i + 1 < len(order) else None
+            wants = getattr(self.blocks[order[i + 1].block], "wants_scaled", None) if i + 1 < len(order) and history is None else None
             leave = wants(T) if wants is not None and getattr(block, "leaves_for_next", False) else None
             if leave is not None:
                 h, pending = block.forward(h, pending, ctx, cache, leave=leave)
             else:
                 h, pending = block.forward(h, pending, ctx, cache)
+            if history is not None:
+                if pending is not None:        # the entry's result has to be complete before it is mixed
+                    h = self.stream_mix.settle(h, pending_for(None, pending, self.rt.dtype))
+                    pending = None
+                if h.data_ptr() != history[i + 1].data_ptr():     # a block that did not work in place
+                    history[i + 1].copy_(h)
+                h = self.stream_mix.forward(history, i, out=history[i + 2] if i + 1 < len(order) else None)
             if self.tap is not None:
                 self.tap(i, h if pending is None else self._settled(h, pending))
         if ctx.logit_rows is None or ctx.logit_rows.shape[0] == 0:

@@ -204,3 +204,81 @@ def selective_scan(dt_pre: torch.Tensor, dt_bias: torch.Tensor, u: torch.Tensor,
                                  _size_t(stride), _ptr(q_start), _ptr(q_len), _ptr(state_slot), _ptr(y), T, B, inner, N, int(max_q_len),
                                  _ptr(scratch), _ptr(y_local), _ptr(dt_sum), run, dtype_code(out_dtype), _stream()), "selective_scan")
     return y
+
+
+def memory_state_floats(heads: int, dk: int, dv: int) -> int:
+    """Floats of one request's state of :func:`gated_memory`: [heads][dv + 1][dk rounded up to 8 * a power of two] (the
+    normaliser is one more value channel), then the running maximum of every head; rounded up to whole 16 bytes."""
+    parts = _pow2_parts(dk, 8)
+    _need(parts <= 64, f"keys of {dk} channels are more than the kernel's 512")
+    return (heads * (dv + 1) * parts * 8 + heads + 3) // 4 * 4
+
+
+def gated_memory(proj: torch.Tensor, q_col: int, k_col: int, v_col: int, z_col: int, gate_bias: torch.Tensor, cap: float,
+                 q_scale: float, state: torch.Tensor, q_start: torch.Tensor, q_len: torch.Tensor, state_slot: torch.Tensor,
+                 H: int, dk: int, dv: int, max_q_len: int = 0, runs=None, run_len: Optional[int] = None):
+    """A matrix memory per head with exponential gates, over the rows of every sequence of the step, in order:
+
+        ``li = cap tanh((zi + bi) / cap);  lf = logsigmoid(cap tanh((zf + bf) / cap));  m' = max(lf + m, li)``
+        ``S <- exp(lf + m - m') S + exp(li - m') k v^T;  n <- exp(lf + m - m') n + exp(li - m') k;  m <- m'``
+
+    ``proj`` float32 [T, wide] holds q and k [H dk each] from columns ``q_col`` and ``k_col``, v [H dv] from ``v_col``
+    and the gates' pre-activations zi [H] | zf [H] from ``z_col``; ``gate_bias`` float32 [2 H] = bi | bf; q is
+    multiplied by ``q_scale``.  ``state`` float32 [slots, >= memory_state_floats(H, dk, dv)] holds S, n and (kept by
+    :func:`memory_norm`) m; S and n are moved on by this call.  Returns ``(raw float32 [T, H, dv + 1], m float32 [T, H])``:
+    ``S^T q`` and, as the last number of a head, ``n . q``, and every token's m.  ``max_q_len``, ``runs`` and ``run_len``
+    as for :func:`decay_attention`: long portions go in runs side by side from an empty memory, chained afterwards."""
+    T, wide = proj.shape
+    _gpu(proj, "proj", torch.float32)
+    for col, n in ((q_col, H * dk), (k_col, H * dk), (v_col, H * dv), (z_col, 2 * H)):
+        _need(0 <= col and col + n <= wide, "the operands' columns lie outside the rows")
+    _gpu(gate_bias, "gate_bias", torch.float32, (2 * H,))
+    _need(cap > 0, "the gates' cap must be positive")
+    stride = _state(state)
+    floats = memory_state_floats(H, dk, dv)
+    _need(stride >= floats, "the state is too small")
+    B = _per_seq(q_start, q_len, state_slot)
+    raw = torch.empty(T, H, dv + 1, dtype=torch.float32, device=proj.device)
+    m = torch.empty(T, H, dtype=torch.float32, device=proj.device)
+    scratch = scalars = None
+    run = 0
+    if _in_runs(max_q_len, T, runs):
+        max_q_len = max_q_len or T
+        parts = _pow2_parts(dk, 8)
+        run = run_tokens(T, H * -(-(dv + 1) // (4 * (64 // parts)))) if run_len is None else int(run_len)
+        n_runs = T // run + B
+        scratch = torch.empty(n_runs * H * (dv + 1) * parts * 8, dtype=torch.float32, device=proj.device)
+        scalars = torch.empty(2 * T * H + 3 * n_runs * H, dtype=torch.float32, device=proj.device)
+    _check(state_mixers_lib().ni_gated_memory(_ptr(proj), wide, int(q_col), int(k_col), int(v_col), int(z_col), _ptr(gate_bias),
+                                              _float(cap), _float(q_scale), _ptr(state), _size_t(stride), _ptr(q_start), _ptr(q_len),
+                                              _ptr(state_slot), _ptr(raw), _ptr(m), T, B, H, dk, dv, int(max_q_len), _ptr(scratch),
+                                              _ptr(scalars), run, _stream()), "gated_memory")
+    return raw, m
+
+
+def memory_norm(raw: torch.Tensor, m: torch.Tensor, gate_rows: torch.Tensor, gate_col: int, weight: torch.Tensor, eps: float,
+                state: torch.Tensor, seq_of_token: torch.Tensor, q_start: torch.Tensor, q_len: torch.Tensor,
+                state_slot: torch.Tensor, dk: int, out_dtype: torch.dtype) -> torch.Tensor:
+    """What :func:`gated_memory` left, finished: ``o = raw[..., :dv] / (max(|raw[..., dv]|, exp(-m)) + 1e-6)``, every head
+    divided by its root mean square (``eps``), times ``weight`` [H dv], times ``sigmoid`` of the gate's pre-activations
+    (columns ``gate_col ..`` of ``gate_rows`` float32 [T, wide]); [T, H dv] in ``out_dtype``.  The m of every sequence's
+    last token is kept in ``state`` for the next step."""
+    T, H, dvn = raw.shape
+    dv = dvn - 1
+    _gpu(raw, "raw", torch.float32)
+    _gpu(m, "m", torch.float32, (T, H))
+    _gpu(gate_rows, "gate_rows", torch.float32)
+    _need(gate_rows.shape[0] == T and 0 <= gate_col and gate_col + H * dv <= gate_rows.shape[1], "the gate's columns lie outside its rows")
+    _gpu(weight, "weight", torch.float32, (H * dv,))
+    stride = _state(state)
+    floats = memory_state_floats(H, dk, dv)
+    _need(stride >= floats, "the state is too small")
+    m_off = H * dvn * _pow2_parts(dk, 8) * 8
+    _gpu(seq_of_token, "seq_of_token", torch.int32, (T,))
+    _per_seq(q_start, q_len, state_slot)
+    y = torch.empty(T, H * dv, dtype=out_dtype, device=raw.device)
+    gate = ctypes.c_void_p(gate_rows.data_ptr() + 4 * gate_col)
+    _check(state_mixers_lib().ni_memory_norm(_ptr(raw), _ptr(m), gate, gate_rows.shape[1], _ptr(weight), _ptr(y), _ptr(state),
+                                             _size_t(stride), _size_t(m_off), _ptr(seq_of_token), _ptr(q_start), _ptr(q_len),
+                                             _ptr(state_slot), T, H, dv, _float(eps), dtype_code(out_dtype), _stream()), "memory_norm")
+    return y

@@ -61,11 +61,13 @@ def add_vector(h: torch.Tensor, vec: torch.Tensor) -> torch.Tensor:
 
 def embed_pair_hash(ids: torch.Tensor, positions: torch.Tensor, seq_of_token: torch.Tensor, q_start: torch.Tensor,
                     q_len: torch.Tensor, state_slot: torch.Tensor, last_token: torch.Tensor, table: torch.Tensor,
-                    pairs: torch.Tensor, buckets: int, mul_prev: int, mul_cur: int, scale: float, out: torch.Tensor) -> torch.Tensor:
+                    pairs: Optional[torch.Tensor], buckets: int, mul_prev: int, mul_cur: int, scale: float, out: torch.Tensor,
+                    freq: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``out[t] = table[ids[t]] * scale + pairs[(prev * mul_prev + ids[t] * mul_cur) mod buckets]`` as float32, ``prev``
     the token before ``ids[t]`` in its sequence; a sequence's first token (position 0) takes row ``buckets``.
     ``last_token`` int32 [slots, 1] holds, per state slot, the last token of the sequence so far: it serves the first
-    row of a portion and is moved on by this call."""
+    row of a portion and is moved on by this call.  ``pairs`` None: no second table.  ``freq`` float32 [(d + 1) // 2]:
+    a sinusoid of the position is added, column 2i ``sin(position * freq[i])`` and column 2i + 1 the cosine."""
     T = ids.shape[0]
     B = q_start.shape[0]
     vocab, d = table.shape
@@ -76,12 +78,15 @@ def embed_pair_hash(ids: torch.Tensor, positions: torch.Tensor, seq_of_token: to
     _need(last_token.is_cuda and last_token.dtype == torch.int32 and last_token.is_contiguous() and last_token.dim() == 2
           and last_token.shape[1] == 1, "last_token must be int32 [slots, 1] on the GPU")
     _gpu(table, "table")
-    _gpu(pairs, "pairs", table.dtype, (buckets + 1, d))
+    if pairs is not None:
+        _gpu(pairs, "pairs", table.dtype, (buckets + 1, d))
+    if freq is not None:
+        _gpu(freq, "freq", torch.float32, ((d + 1) // 2,))
     _gpu(out, "out", torch.float32, (T, d))
     _check(stream_lib().ni_embed_pair_hash(_ptr(ids), _ptr(positions), _ptr(seq_of_token), _ptr(q_start), _ptr(q_len),
                                            _ptr(state_slot), _ptr(last_token), _ptr(table), _ptr(pairs), _ptr(out), T, B, d, vocab,
                                            int(buckets), ctypes.c_longlong(mul_prev), ctypes.c_longlong(mul_cur), _float(scale),
-                                           dtype_code(table.dtype), _stream()), "embed_pair_hash")
+                                           _ptr(freq), dtype_code(table.dtype), _stream()), "embed_pair_hash")
     return out
 
 
@@ -135,6 +140,73 @@ def add_rmsnormed(h: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, eps: f
     _gpu(weight, "weight", torch.float32, (d,))
     _check(stream_lib().ni_add_rmsnormed(_ptr(h), _ptr(y), _ptr(weight), T, d, _float(eps), _stream()), "add_rmsnormed")
     return h
+
+
+def rmsnorm_cols(rows: torch.Tensor, col: int, weight: torch.Tensor, eps: float, out_dtype: torch.dtype) -> torch.Tensor:
+    """``x / sqrt(mean(x^2) + eps) * weight`` over the columns ``col .. col + len(weight)`` of ``rows`` float32 [T, wide]
+    (some of a stacked product's accumulators); [T, len(weight)] in ``out_dtype``."""
+    T, wide = rows.shape
+    n = weight.shape[0]
+    _gpu(rows, "rows", torch.float32)
+    _gpu(weight, "weight", torch.float32, (n,))
+    _need(0 <= col and col + n <= wide, "the columns lie outside the rows")
+    y = torch.empty(T, n, dtype=out_dtype, device=rows.device)
+    src = ctypes.c_void_p(rows.data_ptr() + 4 * col)
+    _check(stream_lib().ni_rmsnorm_cols(src, wide, _ptr(weight), _ptr(y), T, n, _float(eps), dtype_code(out_dtype), _stream()), "rmsnorm_cols")
+    return y
+
+
+def depth_mix(history: torch.Tensor, weights: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """``out[t] = sum_j weights[j] * history[j, t]``: a weighted sum of earlier states of the stream.  ``history``
+    float32 [n, T, d] (contiguous), ``weights`` float32 [n], ``out`` float32 [T, d]."""
+    n, T, d = history.shape
+    _gpu(history, "history", torch.float32)
+    _gpu(weights, "weights", torch.float32, (n,))
+    _gpu(out, "out", torch.float32, (T, d))
+    _check(stream_lib().ni_depth_mix(_ptr(history), _ptr(weights), _ptr(out), n, T, d, _stream()), "depth_mix")
+    return out
+
+
+def poly_norm(z: torch.Tensor, coef: torch.Tensor, eps: float, out_dtype: torch.dtype) -> torch.Tensor:
+    """``a N(z) + b N(z^2) + c N(z^3) + e`` row by row, ``N(u) = u / sqrt(mean(u^2) + eps)``, powers element by element;
+    ``z`` float32 [T, n], ``coef`` float32 [4] = (a, b, c, e); the result in ``out_dtype``."""
+    T, n = z.shape
+    _gpu(z, "z", torch.float32)
+    _gpu(coef, "coef", torch.float32, (4,))
+    y = torch.empty(T, n, dtype=out_dtype, device=z.device)
+    _check(stream_lib().ni_poly_norm(_ptr(z), _ptr(coef), _ptr(y), T, n, _float(eps), dtype_code(out_dtype), _stream()), "poly_norm")
+    return y
+
+
+def scale_(x: torch.Tensor, factor: float) -> torch.Tensor:
+    """``x *= factor`` in place (float32)."""
+    _gpu(x, "x", torch.float32)
+    _check(stream_lib().ni_scale(_ptr(x), _float(factor), _size_t(x.numel()), _stream()), "scale")
+    return x
+
+
+def gate_heads(o: torch.Tensor, gate_rows: torch.Tensor, gate_col: int, out_dtype: torch.dtype) -> torch.Tensor:
+    """``y[t, h * dv + c] = o[h, t, c] * sigmoid(gate[t, h * dv + c])``: ``o`` float32 [H, T, dv] (head by head), the
+    gate's pre-activations the columns ``gate_col ..`` of ``gate_rows`` float32 [T, wide]; y [T, H * dv] in ``out_dtype``."""
+    H, T, dv = o.shape
+    _gpu(o, "o", torch.float32)
+    _gpu(gate_rows, "gate_rows", torch.float32)
+    _need(gate_rows.shape[0] == T and 0 <= gate_col and gate_col + H * dv <= gate_rows.shape[1], "the gate's columns lie outside its rows")
+    y = torch.empty(T, H * dv, dtype=out_dtype, device=o.device)
+    gate = ctypes.c_void_p(gate_rows.data_ptr() + 4 * gate_col)
+    _check(stream_lib().ni_gate_heads(_ptr(o), gate, gate_rows.shape[1], _ptr(y), T, H, dv, dtype_code(out_dtype), _stream()), "gate_heads")
+    return y
+
+
+def heads_apart(x: torch.Tensor, H: int, n: int) -> torch.Tensor:
+    """``y[h, t, c] = x[t, h * n + c]`` for the first ``H * n`` columns of ``x`` [T, wide]: every head's rows together,
+    as a product per head reads them."""
+    T, wide = x.shape
+    _gpu(x, "x")
+    _need(H * n <= wide, "more heads than the rows hold")
+    y = torch.empty(H, T, n, dtype=x.dtype, device=x.device)
+    _check(stream_lib().ni_heads_apart(_ptr(x), wide, _ptr(y), T, H, n, dtype_code(x.dtype), _stream()), "heads_apart")
+    return y
 
 
 # ------------------------------------------------------------------ router and experts
@@ -302,17 +374,26 @@ def kv_store(qkv: torch.Tensor, k_off: int, v_off: int, slot_mapping: torch.Tens
 
 def qk_norm_rope_store(proj: torch.Tensor, positions: torch.Tensor, slot_mapping: Optional[torch.Tensor],
                        q_norm: Optional[torch.Tensor], k_norm: Optional[torch.Tensor], eps: float, freq: Optional[torch.Tensor],
-                       amplitude: float, q_out: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor, H: int) -> torch.Tensor:
+                       amplitude: float, q_out: Optional[torch.Tensor], kpool: torch.Tensor, vpool: torch.Tensor, H: int,
+                       values_are_keys: bool = False, col: int = 0) -> Optional[torch.Tensor]:
     """From ``proj`` float32 [T, H*dk + G*dk + G*dv] (q | k | v as projected): the RMS norm over a token's WHOLE
     query projection and over its whole key projection (weights ``q_norm`` [H*dk], ``k_norm`` [G*dk]; None: no norm),
     then the rotation of the first ``2 * len(freq)`` channels of every head, channel c with channel c + len(freq), by
     ``position * freq[c]`` with cos and sin times ``amplitude`` (``freq`` None: no rotation), all in float32.  Queries
-    go to ``q_out`` [T, H*dk], keys and values into their page slots (``slot_mapping`` None: nothing is stored)."""
-    T, width = proj.shape
+    go to ``q_out`` [T, H*dk], keys and values into their page slots (``slot_mapping`` None: nothing is stored).
+    ``values_are_keys``: ``proj`` is q | k alone and the keys as projected, before their norm, are stored as the values.
+    ``H`` may be 0 (``q_out`` None): keys alone, and values may have no channels.  ``col``: the projections are the
+    columns from ``col`` on of wider rows."""
+    T, wide = proj.shape
+    width = (H + kpool.shape[1]) * kpool.shape[3] + (0 if values_are_keys else kpool.shape[1] * vpool.shape[3])
+    _need(0 <= col and col + width <= wide, "the projections lie outside the rows")
+    if col == 0:
+        width = wide
     pages, G, ps, dk = kpool.shape
     dv = vpool.shape[3]
     _gpu(proj, "proj", torch.float32)
-    _need(width == (H + G) * dk + G * dv, "proj is not q | k | v of these sizes")
+    _need(width == (H + G) * dk + (0 if values_are_keys else G * dv), "proj is not q | k | v of these sizes")
+    _need(not values_are_keys or dv == dk, "values that are the keys have the keys' size")
     _gpu(positions, "positions", torch.int32, (T,))
     if slot_mapping is not None:
         _gpu(slot_mapping, "slot_mapping", torch.int32, (T,))
@@ -327,11 +408,13 @@ def qk_norm_rope_store(proj: torch.Tensor, positions: torch.Tensor, slot_mapping
         _need(0 < rot <= dk, f"{rot} rotated channels do not fit a head of {dk}")
     _gpu(kpool, "kpool")
     _gpu(vpool, "vpool", kpool.dtype, (pages, G, ps, dv))
-    _gpu(q_out, "q_out", kpool.dtype, (T, H * dk))
-    _check(bias_attention_lib().ni_qk_norm_rope_store(_ptr(proj), width, _ptr(positions), _ptr(slot_mapping), _ptr(q_norm),
+    if H > 0 or q_out is not None:
+        _gpu(q_out, "q_out", kpool.dtype, (T, H * dk))
+    src = ctypes.c_void_p(proj.data_ptr() + 4 * col)
+    _check(bias_attention_lib().ni_qk_norm_rope_store(src, wide, _ptr(positions), _ptr(slot_mapping), _ptr(q_norm),
                                                       _ptr(k_norm), _float(eps), _ptr(freq), rot, _float(amplitude), _ptr(q_out),
-                                                      _ptr(kpool), _ptr(vpool), T, H, G, dk, dv, ps, dtype_code(kpool.dtype),
-                                                      _stream()), "qk_norm_rope_store")
+                                                      _ptr(kpool), _ptr(vpool), T, H, G, dk, dv, ps, int(bool(values_are_keys)),
+                                                      dtype_code(kpool.dtype), _stream()), "qk_norm_rope_store")
     return q_out
 
 

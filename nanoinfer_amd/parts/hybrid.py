@@ -159,6 +159,54 @@ def distance_rows(rows: int, far: float, distances: int) -> np.ndarray:
     return out
 
 
+class PagedSoftmax:
+    """Causal softmax attention of ``H`` query heads on ``G`` key/value heads over pages, as the kernels of
+    ``csrc/bias_attention.hip`` compute it: ``score = q . k * scale * temp(i) + bias[i - j, head]``, scores, weights and
+    both products in float32.  Holds the sizes, the constants and the kernels' tile sizes; a mixer calls it with its
+    queries and the pools it reads (keys and values may be the same pool)."""
+
+    def __init__(self, H: int, G: int, dk: int, dv: int, scale: float, temp_coef: float = 0.0, temp_every: int = 0,
+                 bias: Optional[torch.Tensor] = None):
+        if H % G:
+            raise ValueError(f"{H} query heads do not divide into {G} kv heads")
+        self.H, self.G, self.dk, self.dv = H, G, dk, dv
+        self.scale, self.temp_coef, self.temp_every, self.bias = float(scale), float(temp_coef), int(temp_every), bias
+        group = H // G
+        self.heads_per_chunk = min(group, K.bias_attention_rows())
+        self.tile_tokens = max(1, K.bias_attention_rows() // self.heads_per_chunk)
+        K.bias_attention_lib()
+        # steps with portions of prompts: larger tiles on the matrix cores, where the kernel takes these sizes
+        wide = K.bias_attention_mfma_rows(dk, dv)
+        self.wide_heads = min(group, wide) if wide else 0
+        self.wide_tokens = max(1, wide // self.wide_heads) if wide else 0
+
+    def __call__(self, qkv, ctx, kpool, vpool, block_table, window: Optional[int] = None, keep_first: int = 0, out_scale: float = 1.0):
+        T = qkv.shape[0]
+        out = torch.empty(T, self.H * self.dv, dtype=qkv.dtype, device=qkv.device)
+        if self.wide_heads and ctx.max_q_len >= K.BIAS_ATTENTION_MFMA_FROM:
+            tiles = ctx.q_tiles(self.wide_tokens)
+            if tiles is None:
+                raise K.KernelError("this step was recorded without the tiles of its tokens")
+            return K.bias_attention_mfma(qkv, kpool, vpool, block_table, tiles, ctx.positions, self.bias, out, self.H,
+                                         self.scale, self.temp_coef, self.temp_every, self.wide_heads, window, keep_first, out_scale)
+        tiles = ctx.q_tiles(self.tile_tokens)
+        if tiles is None:
+            raise K.KernelError("this step was recorded without the tiles of its tokens")
+        chunks = -(-(self.H // self.G) // self.heads_per_chunk)
+        # a step of single tokens has tiles of one token: its rows are the heads of a chunk, four a wavefront
+        rows = min(self.tile_tokens, ctx.max_q_len) * self.heads_per_chunk
+        # all four wavefronts stage the keys and values, also where fewer of them have rows; the keys are cut into
+        # runs by the wavefronts that have rows
+        waves = 4
+        # with a window a tile walks the kept first keys, the window and its own tokens, in whole tiles of 64 keys
+        max_keys = ctx.max_context if window is None else min(ctx.max_context, window + keep_first + self.tile_tokens + 128)
+        runs = K.bias_attention_runs(tiles.shape[0], self.G, chunks, max_keys, min(4, -(-rows // 4)))
+        ws = ctx.workspace(T * self.H * runs * (self.dv + 2)) if runs > 1 else None
+        return K.bias_attention(qkv, kpool, vpool, block_table, tiles, ctx.positions, self.bias, out, self.H,
+                                self.scale, self.temp_coef, self.temp_every, self.heads_per_chunk, runs, ws, waves, window,
+                                keep_first, out_scale)
+
+
 @register_part("mixer", "bias_attention")
 class BiasAttention(Part):
     """Causal softmax attention with grouped heads and no rotation: positions enter through a learned bias
@@ -192,23 +240,23 @@ class BiasAttention(Part):
         self.scale = float(p["scale"])
         self.temp_coef = 0.0 if p.get("temp_coef") is None else float(p["temp_coef"])
         self.temp_every = 0 if p.get("temp_coef") is None else int(p["temp_every"])
-        self.w_qkv = rt.weight("|".join((names["q"], names["k"], names["v"])),
-                               torch.cat([weights["q"], weights["k"], weights["v"]], dim=0))
+        self.w_qkv = self._stacked_projection(names, weights, rt)
         self.w_o = rt.weight(names["o"], weights["o"])
-        self.bias = None
-        if "bias" in names:
-            # the learned rows laid out by distance, once: the kernel then looks a score's bias up without a logarithm
-            rows = distance_rows(int(p["bias_rows"]), float(p["bias_far"]), int(p["max_positions"]))
-            table = weights["bias"].to(torch.float32)[torch.from_numpy(rows)]
-            self.bias = table.to(rt.device).contiguous()
-        group = self.H // self.G
-        self.heads_per_chunk = min(group, K.bias_attention_rows())
-        self.tile_tokens = max(1, K.bias_attention_rows() // self.heads_per_chunk)
-        K.bias_attention_lib()
-        # steps with portions of prompts: larger tiles on the matrix cores, where the kernel takes these sizes
-        wide = K.bias_attention_mfma_rows(self.dk, self.dv)
-        self.wide_heads = min(group, wide) if wide else 0
-        self.wide_tokens = max(1, wide // self.wide_heads) if wide else 0
+        self.bias = self._bias_table(p, names, weights, rt)
+        self.core = PagedSoftmax(self.H, self.G, self.dk, self.dv, self.scale, self.temp_coef, self.temp_every, self.bias)
+
+    def _stacked_projection(self, names, weights, rt):
+        """The matrix of the part's first product: q | k | v (a subclass may stack others)."""
+        return rt.weight("|".join((names["q"], names["k"], names["v"])), torch.cat([weights["q"], weights["k"], weights["v"]], dim=0))
+
+    def _bias_table(self, p, names, weights, rt) -> Optional[torch.Tensor]:
+        """float32 [distances, H] on the device: what is added to a score at every distance (None: nothing)."""
+        if "bias" not in names:
+            return None
+        # the learned rows laid out by distance, once: the kernel then looks a score's bias up without a logarithm
+        rows = distance_rows(int(p["bias_rows"]), float(p["bias_far"]), int(p["max_positions"]))
+        table = weights["bias"].to(torch.float32)[torch.from_numpy(rows)]
+        return table.to(rt.device).contiguous()
 
     def cache_need(self) -> CacheNeed:
         return CacheNeed(kv=KVNeed(self.G, self.dk, None, self.dv))
@@ -223,30 +271,7 @@ class BiasAttention(Part):
         """The queries in the first ``H * dk`` columns of ``qkv`` over the keys and values of the cache: [T, H * dv] in
         the compute type.  ``window`` n: a query sees its last n keys and the sequence's first ``keep_first``;
         ``out_scale`` multiplies the result."""
-        T = qkv.shape[0]
-        out = torch.empty(T, self.H * self.dv, dtype=qkv.dtype, device=qkv.device)
-        if self.wide_heads and ctx.max_q_len >= K.BIAS_ATTENTION_MFMA_FROM:
-            tiles = ctx.q_tiles(self.wide_tokens)
-            if tiles is None:
-                raise K.KernelError("this step was recorded without the tiles of its tokens")
-            return K.bias_attention_mfma(qkv, cache.kpool, cache.vpool, cache.block_table, tiles, ctx.positions, self.bias, out, self.H,
-                                         self.scale, self.temp_coef, self.temp_every, self.wide_heads, window, keep_first, out_scale)
-        tiles = ctx.q_tiles(self.tile_tokens)
-        if tiles is None:
-            raise K.KernelError("this step was recorded without the tiles of its tokens")
-        chunks = -(-(self.H // self.G) // self.heads_per_chunk)
-        # a step of single tokens has tiles of one token: its rows are the heads of a chunk, four a wavefront
-        rows = min(self.tile_tokens, ctx.max_q_len) * self.heads_per_chunk
-        # all four wavefronts stage the keys and values, also where fewer of them have rows; the keys are cut into
-        # runs by the wavefronts that have rows
-        waves = 4
-        # with a window a tile walks the kept first keys, the window and its own tokens, in whole tiles of 64 keys
-        max_keys = ctx.max_context if window is None else min(ctx.max_context, window + keep_first + self.tile_tokens + 128)
-        runs = K.bias_attention_runs(tiles.shape[0], self.G, chunks, max_keys, min(4, -(-rows // 4)))
-        ws = ctx.workspace(T * self.H * runs * (self.dv + 2)) if runs > 1 else None
-        return K.bias_attention(qkv, cache.kpool, cache.vpool, cache.block_table, tiles, ctx.positions, self.bias, out, self.H,
-                                self.scale, self.temp_coef, self.temp_every, self.heads_per_chunk, runs, ws, waves, window,
-                                keep_first, out_scale)
+        return self.core(qkv, ctx, cache.kpool, cache.vpool, cache.block_table, window, keep_first, out_scale)
 
 
 # ------------------------------------------------------------------ gated delta rule, a decay per key channel

@@ -580,8 +580,8 @@ class PreNormBlock(Block):
 @register_part("head", "linear")
 class LinearHead(Part):
     """``logits = x . W^T`` in float32 output (src/model/llama.cpp:383-386).  params: vocab_size,
-    hidden_size.  weights: weight [vocab, hidden]; a tied head names the embedding's tensor and
-    shares its device buffer."""
+    hidden_size, scale (default 1: the float32 logits are multiplied by it).  weights: weight [vocab, hidden];
+    a tied head names the embedding's tensor and shares its device buffer."""
 
     graph_safe = True
     writes_into = True       # ``forward`` takes ``out=``: float32 [R, vocab] to write the logits into
@@ -595,6 +595,8 @@ class LinearHead(Part):
         self.vocab_size = int(spec.params["vocab_size"])
         # the large matrix is streamed as stored: re-tiling gains nothing at its size and would double it
         self.weight = rt.matrix(spec.weights["weight"], weights["weight"])
+        self.scale = float(spec.params.get("scale", 1.0))
 
     def forward(self, x: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-        return K.linear(x, self.weight, out_dtype=torch.float32, out=out)
+        logits = K.linear(x, self.weight, out_dtype=torch.float32, out=out)
+        return logits if self.scale == 1.0 else K.scale_(logits, self.scale)

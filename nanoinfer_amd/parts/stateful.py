@@ -28,8 +28,11 @@ def _up4(n: int) -> int:
 class PairHashEmbedding(Part):
     """``h[t] = E[id[t]] * scale + P[(prev * mul_prev + id[t] * mul_cur) mod buckets]``: a second table is read by a
     hash of the pair (token before, token); a sequence's first token takes the row behind the buckets.  The token
-    before a portion's first is the last token of the sequence so far, kept per request in a state slot.
-    params: vocab_size, hidden_size, scale, buckets, mul_prev, mul_cur.
+    before a portion's first is the last token of the sequence so far, kept per request in a state slot.  With
+    ``sinusoid_base`` b a vector of the position p is added as well: column 2i ``sin(p * b^(-2i / hidden))``, column
+    2i + 1 the cosine of the same angle (frequencies worked out in float64 and rounded once, the angle a float32 product).
+    params: vocab_size, hidden_size, scale, buckets, mul_prev, mul_cur (``buckets`` None and no ``pairs``: no second
+    table), sinusoid_base (None: none).
     weights: weight [vocab, hidden], pairs [buckets + 1, hidden]."""
 
     graph_safe = True
@@ -38,17 +41,26 @@ class PairHashEmbedding(Part):
     @classmethod
     def weight_requests(cls, spec):
         p, w = spec.params, spec.weights
-        return [WeightRequest(w["weight"], (p["vocab_size"], p["hidden_size"])),
-                WeightRequest(w["pairs"], (p["buckets"] + 1, p["hidden_size"]))]
+        out = [WeightRequest(w["weight"], (p["vocab_size"], p["hidden_size"]))]
+        if "pairs" in w:
+            out.append(WeightRequest(w["pairs"], (p["buckets"] + 1, p["hidden_size"])))
+        return out
 
     def __init__(self, spec, weights, rt):
         super().__init__(spec, weights, rt)
         p = spec.params
         self.hidden_size = int(p["hidden_size"])
         self.scale = float(p.get("scale", 1.0))
-        self.buckets, self.mul_prev, self.mul_cur = int(p["buckets"]), int(p["mul_prev"]), int(p["mul_cur"])
         self.weight = rt.matrix(spec.weights["weight"], weights["weight"])
-        self.pairs = rt.matrix(spec.weights["pairs"], weights["pairs"])
+        self.pairs, self.buckets, self.mul_prev, self.mul_cur = None, 0, 0, 0
+        if "pairs" in spec.weights:
+            self.buckets, self.mul_prev, self.mul_cur = int(p["buckets"]), int(p["mul_prev"]), int(p["mul_cur"])
+            self.pairs = rt.matrix(spec.weights["pairs"], weights["pairs"])
+        self.freq = None
+        if p.get("sinusoid_base") is not None:
+            d, base = self.hidden_size, float(p["sinusoid_base"])
+            freq = torch.tensor([base ** (-2.0 * i / d) for i in range((d + 1) // 2)], dtype=torch.float64)
+            self.freq = freq.to(torch.float32).to(rt.device)
 
     def cache_need(self) -> CacheNeed:
         return CacheNeed(state=StateNeed((1,), torch.int32))
@@ -59,7 +71,7 @@ class PairHashEmbedding(Part):
         out = torch.empty(token_ids.shape[0], self.hidden_size, dtype=torch.float32, device=self.rt.device)
         seq = ctx.per_seq
         return K.embed_pair_hash(token_ids, ctx.positions, ctx.seq_of_token, seq.q_start, seq.q_len, seq.state_slot, cache.state,
-                                 self.weight, self.pairs, self.buckets, self.mul_prev, self.mul_cur, self.scale, out)
+                                 self.weight, self.pairs, self.buckets, self.mul_prev, self.mul_cur, self.scale, out, freq=self.freq)
 
 
 # ------------------------------------------------------------------ softmax attention in a window that keeps the first tokens

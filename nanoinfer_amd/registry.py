@@ -32,7 +32,7 @@ class Architecture:
 ARCHITECTURES: Dict[str, Architecture] = {}
 
 # one table per family of parts; a part class is looked up by the ``kind`` of its spec
-PART_FAMILIES = ("embedding", "norm", "position", "mixer", "feed_forward", "block", "head", "token_input", "pass_input")
+PART_FAMILIES = ("embedding", "norm", "position", "mixer", "feed_forward", "block", "head", "token_input", "pass_input", "stream_mix")
 PARTS: Dict[str, Dict[str, type]] = {family: {} for family in PART_FAMILIES}
 
 

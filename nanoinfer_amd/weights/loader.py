@@ -51,6 +51,8 @@ def expected_tensors(spec: ModelSpec) -> Dict[str, Tuple[int, ...]]:
         requests += get_part("block", b.kind).weight_requests(b)
     if spec.pass_input is not None:
         requests += get_part("pass_input", spec.pass_input.kind).weight_requests(spec.pass_input)
+    if spec.stream_mix is not None:
+        requests += get_part("stream_mix", spec.stream_mix.kind).weight_requests(spec.stream_mix)
     requests += get_part("norm", spec.final_norm.kind).weight_requests(spec.final_norm)
     requests += get_part("head", spec.head.kind).weight_requests(spec.head)
     out: Dict[str, Tuple[int, ...]] = {}

@@ -424,15 +424,46 @@ def fusavik_config(layers: int, vocab: int, like: dict) -> dict:
             "norm": {"eps": 1e-5}, "layers": [dict(pattern[i % 2], mlp=routed) for i in range(layers)]}
 
 
+def ruludra_config(layers: int, vocab: int, like: dict) -> dict:
+    """A Ruludra model whose layers have the sizes of a Llama shape's, four kinds in turn: a matrix memory with
+    exponential gates (width / 128 heads with keys of 64 and values of 128, the sizes of the Fusavik shape's decay
+    attention; no feed-forward), attention whose values are its keys (the shape's heads and head size, a window of 1,024,
+    a penalty by distance and a query factor), attention over a latent of 256 numbers a token (the shape's heads and head
+    size for keys and values, queries through a latent of half the width, a window of 1,024), and a second such layer
+    that reads the latents of the one before; the last three with the shape's dense feed-forward."""
+    width, ff, hd = like["hidden_size"], like["intermediate_size"], like["head_dim"]
+    heads = like["num_attention_heads"]
+    memory = {"type": "mlstm", "mixer": {"heads": width // 128, "dim": 64, "vdim": 128, "gate_cap": 15.0}}
+    keyed = {"type": "attention", "mixer": {"heads": heads, "kv_heads": like["num_key_value_heads"], "dim": hd, "vdim": hd,
+                                            "scale": hd ** -0.5, "mask": {"size": 1024}, "q_temp": {"coef": 0.1, "every": 1024}}}
+    latent = {"heads": heads, "dim": hd, "vdim": hd, "q_rank": width // 2, "kv_rank": 256, "scale": hd ** -0.5, "mask": {"size": 1024}}
+    dense = {"kind": "dense", "ff": ff}
+    out = []
+    for i in range(layers):
+        if i % 4 == 0:
+            out.append(dict(memory, mlp=None))
+        elif i % 4 == 1:
+            out.append(dict(keyed, mlp=dense))
+        elif i % 4 == 2:
+            out.append({"type": "latent_attention", "mixer": dict(latent), "mlp": dense})
+        else:
+            out.append({"type": "latent_attention", "mixer": dict(latent, kv_from=i - 1), "mlp": dense})
+    return {"architecture": "Ruludra", "vocab": vocab, "width": width,
+            "embedding": {"bigram": {"buckets": 16381, "mul_prev": 8191, "mul_cur": 31}}, "norm": {"eps": 1e-5},
+            "logit_scale": float(width) ** -0.5, "layers": out}
+
+
 def hybrid(args) -> int:
     """``--workload hybrid``: prefill of one prompt and decode steps of the Zekalorn shape above and of the Llama
     shape of equal depth, one JSON line with both.  ``--workload stateful``: the same of the Fusavik shape above
-    beside the Zekalorn shape (the framework's other model with mixers that keep a state and routed experts)."""
+    beside the Zekalorn shape (the framework's other model with mixers that keep a state and routed experts).
+    ``--workload latent``: the same of the Ruludra shape above beside the Fusavik shape (the framework's other model
+    with attention in a window, a matrix memory a head and a pair-hash embedding)."""
     import torch
     torch.cuda.set_device(0)
     layers = args.layers or 8
     prompt, batch = args.prompt_len, args.batch
-    first = "fusavik" if args.workload == "stateful" else "zekalorn"
+    first = {"stateful": "fusavik", "latent": "ruludra"}.get(args.workload, "zekalorn")
     out = {"metric": f"{args.workload}_decode_tokens_per_s", "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
            "higher_is_better": True, "dtype": args.dtype, "data": "synthetic token ids, random-init weights",
            "config": {"layers": layers, "prompt_len": prompt, "global_batch": batch, "shape": args.shape,
@@ -442,6 +473,8 @@ def hybrid(args) -> int:
               "llama": dict(like, num_hidden_layers=layers, max_position_embeddings=prompt + 2048)}
     if args.workload == "stateful":
         shapes = {"fusavik": fusavik_config(layers, 128256, like), "zekalorn": shapes["zekalorn"]}
+    if args.workload == "latent":
+        shapes = {"ruludra": ruludra_config(layers, 128256, like), "fusavik": fusavik_config(layers, 128256, like)}
     for name, cfg in shapes.items():
         if args.only and name != args.only:
             continue
@@ -498,12 +531,14 @@ def main() -> int:
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64 and the further points")
     ap.add_argument("--no-further", action="store_true",
                     help="skip the points beyond the default line's: contexts of 8k and 32k, float32, the 3B shape")
-    ap.add_argument("--only", default=None, choices=["zekalorn", "llama", "fusavik"], help="hybrid, stateful: measure one of the two models")
-    ap.add_argument("--workload", default="steps", choices=["steps", "serving", "hybrid", "stateful"],
+    ap.add_argument("--only", default=None, choices=["zekalorn", "llama", "fusavik", "ruludra"],
+                    help="hybrid, stateful, latent: measure one of the two models")
+    ap.add_argument("--workload", default="steps", choices=["steps", "serving", "hybrid", "stateful", "latent"],
                     help="steps: the decode step and prefill of the result line's contract (default); "
                          "serving: concurrent requests through the engine's scheduler, a line of its own; "
                          "hybrid: prefill and decode of a Zekalorn model at the 1B shape's layer sizes beside the Llama shape; "
-                         "stateful: the same of a Fusavik model beside the Zekalorn one")
+                         "stateful: the same of a Fusavik model beside the Zekalorn one; "
+                         "latent: the same of a Ruludra model beside the Fusavik one")
     ap.add_argument("--requests", type=int, default=64, help="serving: concurrent requests")
     ap.add_argument("--new-tokens", type=int, default=256, help="serving: tokens generated per request")
     ap.add_argument("--min-prompt", type=int, default=128, help="serving: shortest prompt")
@@ -524,7 +559,7 @@ def main() -> int:
         return 2
     if args.workload == "serving":
         return serving(args)
-    if args.workload in ("hybrid", "stateful"):
+    if args.workload in ("hybrid", "stateful", "latent"):
         return hybrid(args)
     args.prefill_chunk = args.prefill_chunk or PREFILL_CHUNK
 

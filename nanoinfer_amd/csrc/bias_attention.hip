@@ -481,7 +481,9 @@ bias_attention_mfma_kernel(const T* __restrict__ qkv, int row_stride, const T* _
     const int dkp = dk + 4, dvp = dv + 4;         // strides that spread the sixteen rows of a read over the banks
     float* Qs = lds;                              // [MROWS][dkp]
     float* Ks = Qs + MROWS * dkp;                 // [KEYS][dkp]
-    float* Vs = Ks + KEYS * dkp;                  // [KEYS][dvp]
+    // keys and values that are one pool (dv = dk) are staged once: the values are read from the keys' tile
+    const bool one_pool = static_cast<const void*>(kpool) == static_cast<const void*>(vpool) && dk == dv;
+    float* Vs = one_pool ? Ks : Ks + KEYS * dkp;  // [KEYS][dvp]
     const int tile = blockIdx.x, g = blockIdx.y, chunk = blockIdx.z;
     const int seq = tiles[4 * tile], first_row = tiles[4 * tile + 1], n_tok = tiles[4 * tile + 2];
     const int first_pos = positions[first_row];
@@ -522,7 +524,7 @@ bias_attention_mfma_kernel(const T* __restrict__ qkv, int row_stride, const T* _
         __syncthreads();                          // the tile before this one has been used by everyone
         // one after the other: both in registers at once would cost this kernel its second wavefront a SIMD
         stage_rows<T>(kpool, Ks, dkp, dk, table, page_size, G, g, k0, last_pos, k_pieces);
-        stage_rows<T>(vpool, Vs, dvp, dv, table, page_size, G, g, k0, last_pos, v_pieces);
+        if (!one_pool) stage_rows<T>(vpool, Vs, dvp, dv, table, page_size, G, g, k0, last_pos, v_pieces);
         __syncthreads();
         if (k0 > wave_last) continue;             // nothing here for this wavefront's rows (it still stages and waits)
         floatx4_t sc[KEYS / 16];
@@ -682,11 +684,16 @@ NI_EXPORT int ni_bias_attention(const void* qkv, int row_stride, const void* kpo
     return NI_LAUNCH_RESULT();
 }
 
-// rows of (token, head) of a tile of the matrix-core kernel; 0 where it does not take these sizes
-NI_EXPORT int ni_bias_attention_mfma_rows(int dk, int dv) {
-    if (dk % 16 || dv % 16 || dk < 16 || dv < 16 || dv > MAX_VCHUNKS * WAVE) return 0;
-    const size_t lds = (static_cast<size_t>(MROWS + KEYS) * (dk + 4) + static_cast<size_t>(KEYS) * (dv + 4)) * sizeof(float);
-    return lds <= 160 * 1024 ? MROWS : 0;
+// staging memory of the matrix-core kernel: queries, a tile of keys and, unless they are the keys' pool, one of values
+static size_t mfma_lds_bytes(int dk, int dv, bool one_pool) {
+    return (static_cast<size_t>(MROWS + KEYS) * (dk + 4) + (one_pool ? 0 : static_cast<size_t>(KEYS) * (dv + 4))) * sizeof(float);
+}
+
+// rows of (token, head) of a tile of the matrix-core kernel; 0 where it does not take these sizes.  `one_pool`: keys
+// and values are the same pool (dv = dk)
+NI_EXPORT int ni_bias_attention_mfma_rows(int dk, int dv, int one_pool) {
+    if (dk % 16 || dv % 16 || dk < 16 || dv < 16 || dv > MAX_VCHUNKS * WAVE || (one_pool && dk != dv)) return 0;
+    return mfma_lds_bytes(dk, dv, one_pool != 0) <= 160 * 1024 ? MROWS : 0;
 }
 
 // tiles of up to 64 rows (tokens * heads of a chunk), no runs: for steps with portions of prompts
@@ -697,9 +704,10 @@ NI_EXPORT int ni_bias_attention_mfma(const void* qkv, int row_stride, const void
                                      float out_scale, int dtype, hipStream_t stream) {
     if (n_tiles <= 0) return 0;
     if (window < 0 || keep_first < 0) return -1;
-    if (!ni_bias_attention_mfma_rows(dk, dv) || H % G || heads_per_chunk < 1 || heads_per_chunk > MROWS) return -1;
+    const bool one_pool = kpool == vpool && dk == dv;
+    if (!ni_bias_attention_mfma_rows(dk, dv, one_pool) || H % G || heads_per_chunk < 1 || heads_per_chunk > MROWS) return -1;
     const int group = H / G;
-    const size_t lds = (static_cast<size_t>(MROWS + KEYS) * (dk + 4) + static_cast<size_t>(KEYS) * (dv + 4)) * sizeof(float);
+    const size_t lds = mfma_lds_bytes(dk, dv, one_pool);
     const int vec = dtype == 0 ? 4 : 8;
     const bool k_pieces = dk % vec == 0 && reinterpret_cast<uintptr_t>(kpool) % 16 == 0;
     const bool v_pieces = dv % vec == 0 && reinterpret_cast<uintptr_t>(vpool) % 16 == 0;

@@ -471,10 +471,11 @@ def bias_attention(qkv: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor, 
 BIAS_ATTENTION_MFMA_FROM = 8      # a step whose longest portion has this many tokens takes the matrix-core kernel
 
 
-def bias_attention_mfma_rows(dk: int, dv: int) -> int:
+def bias_attention_mfma_rows(dk: int, dv: int, one_pool: bool = False) -> int:
     """Rows of (token, head) of a tile of the matrix-core kernel for prompt portions; 0 where it does not take
-    these sizes (both multiples of 16, small enough for its staging memory)."""
-    return int(bias_attention_lib().ni_bias_attention_mfma_rows(int(dk), int(dv)))
+    these sizes (both multiples of 16, small enough for its staging memory).  ``one_pool``: keys and values are the
+    same pool, which is staged once and so may be larger."""
+    return int(bias_attention_lib().ni_bias_attention_mfma_rows(int(dk), int(dv), int(bool(one_pool))))
 
 
 def bias_attention_mfma(qkv: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor, block_table: torch.Tensor,
@@ -496,7 +497,8 @@ def bias_attention_mfma(qkv: torch.Tensor, kpool: torch.Tensor, vpool: torch.Ten
     _gpu(out, "out", qkv.dtype, (T, H * dv))
     _gpu(positions, "positions", torch.int32, (T,))
     _need(H % G == 0 and H * dk <= width, "heads")
-    _need(bias_attention_mfma_rows(dk, dv) > 0, f"keys of {dk} and values of {dv} channels are not taken by the matrix-core kernel")
+    _need(bias_attention_mfma_rows(dk, dv, kpool.data_ptr() == vpool.data_ptr()) > 0,
+          f"keys of {dk} and values of {dv} channels are not taken by the matrix-core kernel")
     _need(1 <= heads_per_chunk <= 64, "heads_per_chunk")
     distances = 0
     if bias is not None:

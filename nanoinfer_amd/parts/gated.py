@@ -127,7 +127,7 @@ class LatentAttention(Part):
         # per head: [dk, rank] for the queries' side, [rank, dv] behind the softmax
         self.uk = rt.matrix(names["uk"], weights["uk"]).view(self.H, self.dk, self.rank)
         self.uv_t = rt.matrix(names["uv"], weights["uv"]).view(self.H, self.dv, self.rank).transpose(1, 2)
-        self.core = PagedSoftmax(self.H, 1, self.rank, self.rank, float(p["scale"]))
+        self.core = PagedSoftmax(self.H, 1, self.rank, self.rank, float(p["scale"]), one_pool=True)
         K.stream_lib()
 
     def cache_need(self) -> CacheNeed:

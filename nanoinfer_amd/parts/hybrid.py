@@ -166,7 +166,7 @@ class PagedSoftmax:
     queries and the pools it reads (keys and values may be the same pool)."""
 
     def __init__(self, H: int, G: int, dk: int, dv: int, scale: float, temp_coef: float = 0.0, temp_every: int = 0,
-                 bias: Optional[torch.Tensor] = None):
+                 bias: Optional[torch.Tensor] = None, one_pool: bool = False):
         if H % G:
             raise ValueError(f"{H} query heads do not divide into {G} kv heads")
         self.H, self.G, self.dk, self.dv = H, G, dk, dv
@@ -176,7 +176,8 @@ class PagedSoftmax:
         self.tile_tokens = max(1, K.bias_attention_rows() // self.heads_per_chunk)
         K.bias_attention_lib()
         # steps with portions of prompts: larger tiles on the matrix cores, where the kernel takes these sizes
-        wide = K.bias_attention_mfma_rows(dk, dv)
+        # (``one_pool``: the caller hands the same pool over as keys and as values, which the kernel then stages once)
+        wide = K.bias_attention_mfma_rows(dk, dv, one_pool)
         self.wide_heads = min(group, wide) if wide else 0
         self.wide_tokens = max(1, wide // self.wide_heads) if wide else 0
 

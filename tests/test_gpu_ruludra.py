@@ -333,7 +333,8 @@ def _plain_scores_softmax(q, k, v, scale, window, penalty, factor, H, G):
 @pytest.mark.parametrize("H,G,dk,page,window,shared,temp", [(6, 2, 16, 8, 75, False, (0.5, 16)), (4, 4, 32, 16, 5, False, None),
                                                              (3, 1, 24, 4, 130, True, None), (2, 1, 64, 16, 64, True, None),
                                                              (5, 5, 16, 8, 1, False, (0.3, 7)), (2, 2, 16, 8, None, False, (1.0, 50)),
-                                                             (7, 1, 48, 16, 140, True, None)])
+                                                             (7, 1, 48, 16, 140, True, None), (2, 1, 256, 16, 100, True, None),
+                                                             (3, 1, 128, 8, 40, True, None)])
 def test_window_edges_far_keys_and_the_distance_penalty_in_both_attention_kernels(H, G, dk, page, window, shared, temp, dtype):
     """The attention alone over scattered pages, with one key a query made to stand out: the key just inside the window,
     the key just outside it, a key far back and keys at the edges of the kernel's tiles of 64.  A key that is wrongly
@@ -389,7 +390,7 @@ def test_window_edges_far_keys_and_the_distance_penalty_in_both_attention_kernel
     for first in (0, 100, 203):
         n = T - first
         for wide in (True, False):
-            rows_per = stream.bias_attention_mfma_rows(dk, dk) if wide else stream.bias_attention_rows()
+            rows_per = stream.bias_attention_mfma_rows(dk, dk, shared) if wide else stream.bias_attention_rows()
             if not rows_per:
                 continue
             heads = min(group, rows_per)

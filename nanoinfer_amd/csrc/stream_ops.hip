@@ -83,14 +83,23 @@ __global__ void embed_pair_hash_kernel(const int32_t* __restrict__ ids, const in
     const T* prow = pairs + static_cast<size_t>(row) * d;
     float* o = out + static_cast<size_t>(t) * d;
     const float pos = static_cast<float>(positions[t]);
-    for (int i = threadIdx.x; i < d; i += blockDim.x) {
-        float v = ld(erow + i) * scale;
-        if (pairs) v += ld(prow + i);
-        if (freq) {
-            const float angle = pos * freq[i / 2];
-            v += (i & 1) ? cosf(angle) : sinf(angle);
+    // a thread takes the two columns that share an angle: one reduction of the angle serves the sine and the cosine
+    for (int p = threadIdx.x; 2 * p < d; p += blockDim.x) {
+        const int i = 2 * p;
+        const bool two = i + 1 < d;
+        float v0 = ld(erow + i) * scale, v1 = two ? ld(erow + i + 1) * scale : 0.f;
+        if (pairs) {
+            v0 += ld(prow + i);
+            if (two) v1 += ld(prow + i + 1);
         }
-        o[i] = v;
+        if (freq) {
+            float sn, cs;
+            sincosf(pos * freq[p], &sn, &cs);
+            v0 += sn;
+            v1 += cs;
+        }
+        o[i] = v0;
+        if (two) o[i + 1] = v1;
     }
 }
 
@@ -297,11 +306,21 @@ poly_norm_kernel(const float* __restrict__ z, const float* __restrict__ coef, T*
     __shared__ float scratch[16];
     const float* row = z + static_cast<size_t>(blockIdx.x) * n;
     float s2 = 0.f, s4 = 0.f, s6 = 0.f;
-    for (int i = threadIdx.x; i < n; i += blockDim.x) {
-        const float v = row[i], v2 = v * v;
-        s2 += v2;
-        s4 += v2 * v2;
-        s6 += v2 * v2 * v2;
+    if (n % 4 == 0 && reinterpret_cast<uintptr_t>(z) % 16 == 0) {        // whole 16-byte pieces
+        for (int i = 4 * threadIdx.x; i < n; i += 4 * blockDim.x) {
+            const float4 q = *reinterpret_cast<const float4*>(row + i);
+            const float a = q.x * q.x, b = q.y * q.y, c = q.z * q.z, e = q.w * q.w;
+            s2 += (a + b) + (c + e);
+            s4 += (a * a + b * b) + (c * c + e * e);
+            s6 += (a * a * a + b * b * b) + (c * c * c + e * e * e);
+        }
+    } else {
+        for (int i = threadIdx.x; i < n; i += blockDim.x) {
+            const float v = row[i], v2 = v * v;
+            s2 += v2;
+            s4 += v2 * v2;
+            s6 += v2 * v2 * v2;
+        }
     }
     s2 = block_sum(s2, scratch);
     s4 = block_sum(s4, scratch);

@@ -581,14 +581,13 @@ NI_EXPORT int ni_selective_scan(const void* dt_pre, const void* dt_bias, const v
 // recurrence kernels leave the raw read-outs [T, H (dv + 1)] (the last of a head is n . q) and m [T, H];
 // memory_norm_kernel divides, norms every head, gates, and keeps the last m of every sequence in the state.
 struct MemoryOperands {
-    float q[DKPT], k[DKPT], v, li, lf;
+    float q[DKPT], k[DKPT], v;
 };
 
 __device__ __forceinline__ float log_sigmoid_f(float x) { return fminf(x, 0.f) - log1pf(expf(-fabsf(x))); }
 
 __device__ __forceinline__ void memory_load(MemoryOperands& o, const float* __restrict__ row, int q_off, int k_off, int v_off,
-                                            int zi_off, int zf_off, float bi, float bf, float cap, float q_scale, int ch, int dk,
-                                            bool whole, bool ones) {
+                                            float q_scale, int ch, int dk, bool whole, bool ones) {
     if (whole) {
         const float4 a = *reinterpret_cast<const float4*>(row + q_off + ch), b = *reinterpret_cast<const float4*>(row + q_off + ch + 4);
         const float4 c = *reinterpret_cast<const float4*>(row + k_off + ch), d = *reinterpret_cast<const float4*>(row + k_off + ch + 4);
@@ -605,9 +604,10 @@ __device__ __forceinline__ void memory_load(MemoryOperands& o, const float* __re
 #pragma unroll
     for (int i = 0; i < DKPT; ++i) o.q[i] *= q_scale;
     o.v = ones ? 1.f : row[v_off];
-    o.li = cap * tanhf((row[zi_off] + bi) / cap);
-    o.lf = log_sigmoid_f(cap * tanhf((row[zf_off] + bf) / cap));
 }
+
+// tokens whose gates a workgroup works out together, one a thread
+constexpr int GATE_TOKENS = 256;
 
 // Token by token from the state (LOCAL false), or a run of RUN tokens from an empty memory whose maximum starts at
 // minus infinity (LOCAL true; the runs' layout is decay_attention_kernel's).  A LOCAL run also leaves, per token, the
@@ -620,6 +620,10 @@ memory_steps_kernel(const float* __restrict__ proj, int stride, int q_col, int k
                     const int32_t* __restrict__ q_len, const int32_t* __restrict__ state_slot, float* __restrict__ out,
                     float* __restrict__ m_out, float* __restrict__ since, float* __restrict__ run_ends, int H, int dk, int dv,
                     int parts, float* __restrict__ runs, int xblocks, int RUN) {
+    // the gates are the same for every column of a head: the workgroup works them out once, GATE_TOKENS tokens at a
+    // time and one a thread (li, lf), one thread walks the maxima (additions and comparisons only), and every thread
+    // again makes its token's two factors exp(lf + m - m') and exp(li - m'), which the columns' lanes then read
+    __shared__ float g_take[GATE_TOKENS], g_keep[GATE_TOKENS], g_m[GATE_TOKENS], g_passed[GATE_TOKENS];
     const int b = blockIdx.z, h = blockIdx.y;
     const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
     const int cols = WAVE / parts;
@@ -629,21 +633,22 @@ memory_steps_kernel(const float* __restrict__ proj, int stride, int q_col, int k
     const int first = run * RUN;
     const int n = LOCAL ? min(q_len[b] - first, RUN) : q_len[b];
     const int dvn = dv + 1;
-    if (c >= dvn || n <= 0) return;               // whole groups of `parts` lanes leave together
+    if (n <= 0) return;                           // the whole workgroup
+    const bool active = c < dvn;                  // a group of `parts` lanes holds a column or none
     const int dkp = parts * DKPT, ch = part * DKPT;
     const size_t heads_floats = static_cast<size_t>(H) * dvn * dkp;
     const size_t run_index = LOCAL ? static_cast<size_t>(q_start[b] / RUN + b + run) : 0;
     const size_t at = (static_cast<size_t>(h) * dvn + c) * dkp + ch;
     float S[DKPT];
-    float m;
-    if (LOCAL) {
 #pragma unroll
-        for (int i = 0; i < DKPT; ++i) S[i] = 0.f;
-        m = -INFINITY;
-    } else {
+    for (int i = 0; i < DKPT; ++i) S[i] = 0.f;
+    float m = -INFINITY;
+    if (!LOCAL) {
         const float* srow = state + static_cast<size_t>(state_slot[b]) * state_stride;
-        const float4 a = *reinterpret_cast<const float4*>(srow + at), d = *reinterpret_cast<const float4*>(srow + at + 4);
-        S[0] = a.x; S[1] = a.y; S[2] = a.z; S[3] = a.w; S[4] = d.x; S[5] = d.y; S[6] = d.z; S[7] = d.w;
+        if (active) {
+            const float4 a = *reinterpret_cast<const float4*>(srow + at), d = *reinterpret_cast<const float4*>(srow + at + 4);
+            S[0] = a.x; S[1] = a.y; S[2] = a.z; S[3] = a.w; S[4] = d.x; S[5] = d.y; S[6] = d.z; S[7] = d.w;
+        }
         m = srow[heads_floats + h];
     }
     const float bi = gate_bias[h], bf = gate_bias[H + h];
@@ -651,39 +656,70 @@ memory_steps_kernel(const float* __restrict__ proj, int stride, int q_col, int k
     const bool whole = dk % DKPT == 0 && ch + DKPT <= dk && stride % 4 == 0 && q_col % 4 == 0 && k_col % 4 == 0;
     const bool idle = ch >= dk;                   // a lane that holds padding only
     const bool ones = c == dv;                    // the normaliser's column
-    const bool scribe = xb == 0 && wave == 0 && lane == 0;     // the one thread of (sequence, head, run) that writes the scalars
+    const bool scribe = xb == 0;                  // the one workgroup of (sequence, head, run) that writes the scalars
     const int t0 = q_start[b] + first;
     float passed = 0.f;                           // sum of lf since the run's start
     MemoryOperands cur, nxt;
-    memory_load(cur, proj + static_cast<size_t>(t0) * stride, q_off, k_off, v_off, zi_off, zf_off, bi, bf, cap, q_scale, ch, dk, whole && !idle, ones);
-    for (int r = 0; r < n; ++r) {
-        if (r + 1 < n)
-            memory_load(nxt, proj + static_cast<size_t>(t0 + r + 1) * stride, q_off, k_off, v_off, zi_off, zf_off, bi, bf, cap, q_scale,
-                        ch, dk, whole && !idle, ones);
-        const float m_new = fmaxf(cur.lf + m, cur.li);
-        const float keep = expf(cur.lf + m - m_new), take = expf(cur.li - m_new) * cur.v;
-        float sum = 0.f;
-        if (!idle) {
-#pragma unroll
-            for (int i = 0; i < DKPT; ++i) {
-                S[i] = keep * S[i] + take * cur.k[i];
-                sum += S[i] * cur.q[i];
+    if (active) memory_load(cur, proj + static_cast<size_t>(t0) * stride, q_off, k_off, v_off, q_scale, ch, dk, whole && !idle, ones);
+    for (int base = 0; base < n; base += GATE_TOKENS) {
+        const int cn = min(n - base, GATE_TOKENS);
+        const int r_own = threadIdx.x;
+        if (r_own < cn) {
+            const float* row = proj + static_cast<size_t>(t0 + base + r_own) * stride;
+            g_take[r_own] = cap * tanhf((row[zi_off] + bi) / cap);                     // li
+            g_keep[r_own] = log_sigmoid_f(cap * tanhf((row[zf_off] + bf) / cap));      // lf
+        }
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            float mm = m, pp = passed;
+            for (int r = 0; r < cn; ++r) {
+                mm = fmaxf(g_keep[r] + mm, g_take[r]);
+                pp += g_keep[r];
+                g_m[r] = mm;
+                g_passed[r] = pp;
             }
         }
-        m = m_new;
-        passed += cur.lf;
-        sum = parts_sum(sum, parts);
-        if (part == 0) out[static_cast<size_t>(t0 + r) * (H * dvn) + h * dvn + c] = sum;
-        if (scribe) {
-            m_out[static_cast<size_t>(t0 + r) * H + h] = m;
-            if (LOCAL) since[static_cast<size_t>(t0 + r) * H + h] = passed;
+        __syncthreads();
+        if (r_own < cn) {
+            const float before = r_own ? g_m[r_own - 1] : m, now = g_m[r_own];
+            const float li = g_take[r_own], lf = g_keep[r_own];
+            g_keep[r_own] = expf(lf + before - now);
+            g_take[r_own] = expf(li - now);
+            if (scribe) {
+                m_out[static_cast<size_t>(t0 + base + r_own) * H + h] = now;
+                if (LOCAL) since[static_cast<size_t>(t0 + base + r_own) * H + h] = g_passed[r_own];
+            }
         }
-        cur = nxt;
+        __syncthreads();
+        if (active) {
+            for (int r = 0; r < cn; ++r) {
+                if (base + r + 1 < n)
+                    memory_load(nxt, proj + static_cast<size_t>(t0 + base + r + 1) * stride, q_off, k_off, v_off, q_scale, ch, dk,
+                                whole && !idle, ones);
+                const float keep = g_keep[r], take = g_take[r] * cur.v;
+                float sum = 0.f;
+                if (!idle) {
+#pragma unroll
+                    for (int i = 0; i < DKPT; ++i) {
+                        S[i] = keep * S[i] + take * cur.k[i];
+                        sum += S[i] * cur.q[i];
+                    }
+                }
+                sum = parts_sum(sum, parts);
+                if (part == 0) out[static_cast<size_t>(t0 + base + r) * (H * dvn) + h * dvn + c] = sum;
+                cur = nxt;
+            }
+        }
+        m = g_m[cn - 1];
+        passed = g_passed[cn - 1];
+        __syncthreads();                          // the next tokens' gates take these places
     }
-    float* dst = LOCAL ? runs + run_index * heads_floats + at : state_out + static_cast<size_t>(state_slot[b]) * state_stride + at;
-    *reinterpret_cast<float4*>(dst) = make_float4(S[0], S[1], S[2], S[3]);
-    *reinterpret_cast<float4*>(dst + 4) = make_float4(S[4], S[5], S[6], S[7]);
-    if (LOCAL && scribe) {
+    if (active) {
+        float* dst = LOCAL ? runs + run_index * heads_floats + at : state_out + static_cast<size_t>(state_slot[b]) * state_stride + at;
+        *reinterpret_cast<float4*>(dst) = make_float4(S[0], S[1], S[2], S[3]);
+        *reinterpret_cast<float4*>(dst + 4) = make_float4(S[4], S[5], S[6], S[7]);
+    }
+    if (LOCAL && scribe && threadIdx.x == 0) {
         run_ends[(run_index * H + h) * 2] = m;
         run_ends[(run_index * H + h) * 2 + 1] = passed;
     }
@@ -723,6 +759,8 @@ memory_carry_kernel(const float* __restrict__ proj, int stride, int q_col, float
                     const float* __restrict__ run_starts, const float* __restrict__ local_max, const float* __restrict__ since,
                     const int32_t* __restrict__ q_start, const int32_t* __restrict__ q_len, float* __restrict__ out,
                     float* __restrict__ m_out, int H, int dk, int dv, int parts, int xblocks, int RUN) {
+    // what a token's own read-out and what the memory at the run's start weigh, once a workgroup and token
+    __shared__ float f_own[GATE_TOKENS], f_before[GATE_TOKENS];
     const int b = blockIdx.z, h = blockIdx.y;
     const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
     const int cols = WAVE / parts;
@@ -732,12 +770,15 @@ memory_carry_kernel(const float* __restrict__ proj, int stride, int q_col, float
     const int first = run * RUN;
     const int n = min(q_len[b] - first, RUN);
     const int dvn = dv + 1;
-    if (c >= dvn || n <= 0) return;
+    if (n <= 0) return;                           // the whole workgroup
+    const bool active = c < dvn;
     const int dkp = parts * DKPT, ch = part * DKPT;
     const size_t run_index = static_cast<size_t>(q_start[b] / RUN + b + run);
     const float* srow = runs + run_index * H * dvn * dkp + (static_cast<size_t>(h) * dvn + c) * dkp + ch;
     float S[DKPT];
-    {
+#pragma unroll
+    for (int i = 0; i < DKPT; ++i) S[i] = 0.f;
+    if (active) {
         const float4 a = *reinterpret_cast<const float4*>(srow), d = *reinterpret_cast<const float4*>(srow + 4);
         S[0] = a.x; S[1] = a.y; S[2] = a.z; S[3] = a.w; S[4] = d.x; S[5] = d.y; S[6] = d.z; S[7] = d.w;
     }
@@ -745,29 +786,40 @@ memory_carry_kernel(const float* __restrict__ proj, int stride, int q_col, float
     const int q_off = q_col + h * dk + ch;
     const bool whole = dk % DKPT == 0 && ch + DKPT <= dk && stride % 4 == 0 && q_col % 4 == 0;
     const bool idle = ch >= dk;
-    const bool scribe = xb == 0 && wave == 0 && lane == 0;
+    const bool scribe = xb == 0;
     const int t0 = q_start[b] + first;
-    for (int r = 0; r < n; ++r) {
-        const float* row = proj + static_cast<size_t>(t0 + r) * stride + q_off;
-        float sum = 0.f;
-        if (!idle) {
-            if (whole) {
-                const float4 a = *reinterpret_cast<const float4*>(row), d = *reinterpret_cast<const float4*>(row + 4);
-                sum = S[0] * a.x + S[1] * a.y + S[2] * a.z + S[3] * a.w + S[4] * d.x + S[5] * d.y + S[6] * d.z + S[7] * d.w;
-            } else {
+    for (int base = 0; base < n; base += GATE_TOKENS) {
+        const int cn = min(n - base, GATE_TOKENS);
+        if (threadIdx.x < cn) {
+            const size_t th = static_cast<size_t>(t0 + base + threadIdx.x) * H + h;
+            const float own = local_max[th], before = since[th] + m0;
+            const float m = fmaxf(before, own);
+            f_own[threadIdx.x] = expf(own - m);
+            f_before[threadIdx.x] = expf(before - m);
+            if (scribe) m_out[th] = m;
+        }
+        __syncthreads();
+        if (active) {
+            for (int r = 0; r < cn; ++r) {
+                const float* row = proj + static_cast<size_t>(t0 + base + r) * stride + q_off;
+                float sum = 0.f;
+                if (!idle) {
+                    if (whole) {
+                        const float4 a = *reinterpret_cast<const float4*>(row), d = *reinterpret_cast<const float4*>(row + 4);
+                        sum = S[0] * a.x + S[1] * a.y + S[2] * a.z + S[3] * a.w + S[4] * d.x + S[5] * d.y + S[6] * d.z + S[7] * d.w;
+                    } else {
 #pragma unroll
-                for (int i = 0; i < DKPT; ++i) sum += ch + i < dk ? S[i] * row[i] : 0.f;
+                        for (int i = 0; i < DKPT; ++i) sum += ch + i < dk ? S[i] * row[i] : 0.f;
+                    }
+                }
+                sum = parts_sum(sum, parts) * q_scale;
+                if (part == 0) {
+                    float* o = out + static_cast<size_t>(t0 + base + r) * (H * dvn) + h * dvn + c;
+                    *o = f_own[r] * *o + f_before[r] * sum;
+                }
             }
         }
-        sum = parts_sum(sum, parts) * q_scale;
-        const size_t th = static_cast<size_t>(t0 + r) * H + h;
-        const float own = local_max[th], before = since[th] + m0;
-        const float m = fmaxf(before, own);
-        if (part == 0) {
-            float* o = out + static_cast<size_t>(t0 + r) * (H * dvn) + h * dvn + c;
-            *o = expf(own - m) * *o + expf(before - m) * sum;
-        }
-        if (scribe) m_out[th] = m;
+        __syncthreads();                          // the next tokens' factors take these places
     }
 }
 

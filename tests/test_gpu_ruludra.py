@@ -449,11 +449,12 @@ def test_matrix_memory_kernels_against_the_plain_recurrence(H, dk, dv, cap, runs
     before left, with gates from shut to wide open (pre-activations far beyond the cap on both sides), so that the
     running maximum rises and the floor ``exp(-m)`` of the divisor is at work early and the normaliser later; against the
     recurrence written out in float64.  Token by token, and in runs that are chained afterwards (sequences of one token,
-    of a run and a bit, of less than a run)."""
+    of a run and a bit, of less than a run).  One size walks a sequence, and one a run, of more tokens than a workgroup
+    works the gates out for at a time."""
     from nanoinfer_amd import kernels as K
     dev = torch.device("cuda")
     g = torch.Generator().manual_seed(2)
-    lens = [37, 1, 150] if not runs else [64, 1, 203]
+    lens = [37, 1, 300 if dv == 48 else 150] if not runs else [64, 1, 650 if H == 3 else 203]
     pad = 3                                          # columns that belong to nobody, before and between the operands
     q_col, k_col = pad, pad + H * dk + 1
     v_col = k_col + H * dk + 2
@@ -489,7 +490,7 @@ def test_matrix_memory_kernels_against_the_plain_recurrence(H, dk, dv, cap, runs
         proj = rows.to(dev)
         raw, mx = K.gated_memory(proj, q_col, k_col, v_col, z_col, bias.to(dev), cap, dk ** -0.5, state, q_start, q_len, slots,
                                  H, dk, dv, max_q_len=max(lens), runs=runs and call < 2,
-                                 run_len=(64 if H == 2 else None) if runs and call < 2 else None)
+                                 run_len=(64 if H == 2 else 300 if H == 3 else None) if runs and call < 2 else None)
         y = K.memory_norm(raw, mx, proj, g_col, norm.to(dev), eps, state, seq_of, q_start, q_len, slots, dk, torch.float32)
         want = np.zeros((T, H * dv))
         for b, (t0, n) in enumerate(zip(starts, lens)):

@@ -404,6 +404,79 @@ NI_EXPORT int ni_heads_apart(const void* x, int x_stride, void* y, int T, int H,
     return NI_LAUNCH_RESULT();
 }
 
+// ---------------------------------------------------------------- rows times the sigmoid of a gate
+//   y[t, j] = x[t, j] * sigmoid(g[t, j])      x [T, n] in the compute type, g float32 rows of stride g_stride
+template <typename T>
+__global__ void gate_rows_kernel(const T* __restrict__ x, const float* __restrict__ g, int g_stride, T* __restrict__ y, int n,
+                                 size_t total) {
+    const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    const size_t t = i / n;
+    const int j = static_cast<int>(i % n);
+    const float gate = 1.0f / (1.0f + expf(-g[t * g_stride + j]));
+    st(y + i, ld(x + i) * gate);
+}
+
+NI_EXPORT int ni_gate_rows(const void* x, const void* g, int g_stride, void* y, int T, int n, int dtype, hipStream_t stream) {
+    const size_t total = static_cast<size_t>(T) * n;
+    if (total == 0) return 0;
+    if (g_stride < n) return -1;
+    if (dtype == 0)
+        gate_rows_kernel<float><<<blocks_of(total, 256), 256, 0, stream>>>((const float*)x, (const float*)g, g_stride, (float*)y, n, total);
+    else
+        gate_rows_kernel<bf16_t><<<blocks_of(total, 256), 256, 0, stream>>>((const bf16_t*)x, (const float*)g, g_stride, (bf16_t*)y, n, total);
+    return NI_LAUNCH_RESULT();
+}
+
+// ---------------------------------------------------------------- pages of a pool, picked through a block table
+//   out[i] = pool[table[pairs[2 i] * width + pairs[2 i + 1]]]      a page is `page_elems` contiguous elements; a page the
+//   table does not hold (< 0) gives zeros
+template <typename T>
+__global__ void gather_pages_kernel(const T* __restrict__ pool, const int32_t* __restrict__ table, int width,
+                                    const int32_t* __restrict__ pairs, T* __restrict__ out, int page_elems) {
+    const int i = blockIdx.x;
+    const int page = table[static_cast<size_t>(pairs[2 * i]) * width + pairs[2 * i + 1]];
+    const T* src = pool + static_cast<size_t>(max(page, 0)) * page_elems;
+    T* dst = out + static_cast<size_t>(i) * page_elems;
+    for (int e = threadIdx.x; e < page_elems; e += blockDim.x) st(dst + e, page >= 0 ? ld(src + e) : 0.f);
+}
+
+NI_EXPORT int ni_gather_pages(const void* pool, const void* table, int width, const void* pairs, void* out, int n_pages,
+                              int page_elems, int dtype, hipStream_t stream) {
+    if (n_pages <= 0 || page_elems <= 0) return 0;
+    if (width < 1) return -1;
+    if (dtype == 0)
+        gather_pages_kernel<float><<<n_pages, 256, 0, stream>>>((const float*)pool, (const int32_t*)table, width, (const int32_t*)pairs,
+                                                                (float*)out, page_elems);
+    else
+        gather_pages_kernel<bf16_t><<<n_pages, 256, 0, stream>>>((const bf16_t*)pool, (const int32_t*)table, width, (const int32_t*)pairs,
+                                                                 (bf16_t*)out, page_elems);
+    return NI_LAUNCH_RESULT();
+}
+
+// ---------------------------------------------------------------- rows of heads, page by page, as pages of heads
+//   y[p][h][s][c] = x[(p * page + s), h * n + c]      (the layout of a pool of keys or values: [page][head][slot][channel])
+template <typename T>
+__global__ void rows_to_pages_kernel(const T* __restrict__ x, T* __restrict__ y, int page, int H, int n, size_t total) {
+    const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    const int c = static_cast<int>(i % n);
+    const int s = static_cast<int>((i / n) % page);
+    const int h = static_cast<int>((i / (static_cast<size_t>(n) * page)) % H);
+    const size_t p = i / (static_cast<size_t>(n) * page * H);
+    y[i] = x[(p * page + s) * (static_cast<size_t>(H) * n) + h * n + c];
+}
+
+NI_EXPORT int ni_rows_to_pages(const void* x, void* y, int n_pages, int page, int H, int n, int dtype, hipStream_t stream) {
+    const size_t total = static_cast<size_t>(n_pages) * page * H * n;
+    if (total == 0) return 0;
+    if (dtype == 0)
+        rows_to_pages_kernel<float><<<blocks_of(total, 256), 256, 0, stream>>>((const float*)x, (float*)y, page, H, n, total);
+    else
+        rows_to_pages_kernel<bf16_t><<<blocks_of(total, 256), 256, 0, stream>>>((const bf16_t*)x, (bf16_t*)y, page, H, n, total);
+    return NI_LAUNCH_RESULT();
+}
+
 // ---------------------------------------------------------------- the router's choice
 // z float32 [T, E]: the `top` largest logits of a row (the lower index on equal logits) and their weights:
 // the softmax among the chosen (`over_all` 0) or the softmax over all E experts, not renormalised (`over_all` 1).

@@ -66,6 +66,12 @@ class Model:
         that its launches depend on device data only (``graph_safe``), never on the host lists."""
         return all(flag_of(p, "graph_safe", False) for p in self._all_parts())
 
+    def eager_portion_from(self) -> Optional[int]:
+        """The fewest tokens of a portion from which on some part wants the step run the ordinary way (it reads the
+        step's host lists then); None: no part does."""
+        asked = [n for n in (getattr(p, "eager_portion_from", None) for p in self._all_parts()) if n is not None]
+        return min(asked) if asked else None
+
     def idempotent(self) -> bool:
         """Whether running the same step twice leaves the caches as running it once does: true of keys
         and values written to their places, not of a per-request state that a part updates in place."""

@@ -251,6 +251,7 @@ class ModelRunner:
     STAGING_BUFFERS = 4           # pinned copies of a recorded step's tables, used in turn
     HISTORY_ROWS = 16             # decode steps launched back to back before the host reads their tokens
     GRAPH_MIN_PORTION = 64        # a shorter prompt portion is not worth a recording
+    _eager_from = None            # a portion of this many tokens is never run from a recording (None: any may be)
     GRAPH_MAX_PORTIONS = 24       # recordings of prompt portions kept (each holds its activations)
     GRAPH_MAX_DECODES = 1024      # recordings of decode steps kept (their logits go to one buffer that all share);
                                   # beyond that the one used longest ago is dropped and its shape recorded again if it returns
@@ -355,6 +356,7 @@ class ModelRunner:
     def _init_graphs(self, use_graphs: bool) -> None:
         import os
         self.use_graphs = bool(use_graphs) and self.model.graph_safe() and not os.environ.get("NANOINFER_NO_GRAPHS")
+        self._eager_from = getattr(self.model, "eager_portion_from", lambda: None)()
         self._recorded: Dict[tuple, _RecordedStep] = {}      # in the order of their last use
         self._recorded_bytes = 0                             # device memory the recordings hold, as measured when each was made
         self._logits_buffer = None                           # float32 [GRAPH_MAX_BATCH, vocabulary]: where recorded steps leave their logits
@@ -554,6 +556,8 @@ class ModelRunner:
         first = entries[0]
         n = len(first.tokens)
         if len(entries) == 1 and n >= self.GRAPH_MIN_PORTION:
+            if self._eager_from is not None and n >= self._eager_from:
+                return None                   # a part reads the host lists of steps with portions this long
             want = list(first.want)
             if want and want != [n - 1]:
                 return None

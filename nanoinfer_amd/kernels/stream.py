@@ -198,6 +198,46 @@ def gate_heads(o: torch.Tensor, gate_rows: torch.Tensor, gate_col: int, out_dtyp
     return y
 
 
+def gate_rows(x: torch.Tensor, gate_rows_: torch.Tensor, gate_col: int, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``y[t, j] = x[t, j] * sigmoid(gate[t, j])``: ``x`` [T, n] in the compute type, the gate's pre-activations the
+    columns ``gate_col ..`` of ``gate_rows_`` float32 [T, wide]; y like x."""
+    T, n = x.shape
+    _gpu(x, "x")
+    _gpu(gate_rows_, "gate_rows", torch.float32)
+    _need(gate_rows_.shape[0] == T and 0 <= gate_col and gate_col + n <= gate_rows_.shape[1], "the gate's columns lie outside its rows")
+    y = torch.empty_like(x) if out is None else out
+    gate = ctypes.c_void_p(gate_rows_.data_ptr() + 4 * gate_col)
+    _check(stream_lib().ni_gate_rows(_ptr(x), gate, gate_rows_.shape[1], _ptr(y), T, n, dtype_code(x.dtype), _stream()), "gate_rows")
+    return y
+
+
+def gather_pages(pool: torch.Tensor, block_table: torch.Tensor, pairs: torch.Tensor) -> torch.Tensor:
+    """Pages of ``pool`` [pages, ...] picked through ``block_table`` int32 [B, width]: ``pairs`` int32 [n, 2] rows of
+    (sequence, index of the page in the sequence's table); [n, ...] like the pool's pages, zeros where the table holds
+    no page."""
+    _gpu(pool, "pool")
+    _gpu(block_table, "block_table", torch.int32)
+    _gpu(pairs, "pairs", torch.int32)
+    _need(pairs.dim() == 2 and pairs.shape[1] == 2 and block_table.dim() == 2, "pairs are rows of (sequence, page index)")
+    n = pairs.shape[0]
+    out = torch.empty((n,) + tuple(pool.shape[1:]), dtype=pool.dtype, device=pool.device)
+    page_elems = pool[0].numel()
+    _check(stream_lib().ni_gather_pages(_ptr(pool), _ptr(block_table), block_table.shape[1], _ptr(pairs), _ptr(out), n, page_elems,
+                                        dtype_code(pool.dtype), _stream()), "gather_pages")
+    return out
+
+
+def rows_to_pages(x: torch.Tensor, page: int, H: int, n: int) -> torch.Tensor:
+    """``y[p, h, s, c] = x[p * page + s, h * n + c]``: rows [pages * page, H * n] of heads side by side as a pool of
+    keys or values, [pages, H, page, n]."""
+    rows, wide = x.shape
+    _gpu(x, "x")
+    _need(wide == H * n and rows % page == 0, "the rows are not whole pages of these heads")
+    y = torch.empty(rows // page, H, page, n, dtype=x.dtype, device=x.device)
+    _check(stream_lib().ni_rows_to_pages(_ptr(x), _ptr(y), rows // page, page, H, n, dtype_code(x.dtype), _stream()), "rows_to_pages")
+    return y
+
+
 def heads_apart(x: torch.Tensor, H: int, n: int) -> torch.Tensor:
     """``y[h, t, c] = x[t, h * n + c]`` for the first ``H * n`` columns of ``x`` [T, wide]: every head's rows together,
     as a product per head reads them."""

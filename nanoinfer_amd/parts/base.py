@@ -128,6 +128,9 @@ class Part:
     # a step more than once (the recording of a step into a HIP graph does) then puts the
     # per-request state back in between.
     idempotent = True
+    # a number of tokens from which on a step with such a portion must run the ordinary way, not from a recording,
+    # because the part then reads the step's host lists (None: recordings of any step are fine)
+    eager_portion_from: Optional[int] = None
 
     @classmethod
     def weight_requests(cls, spec: PartSpec) -> List[WeightRequest]:
@@ -202,6 +205,11 @@ class Block:
 
     def idempotent(self) -> bool:
         return all(flag_of(p, "idempotent", True) for p in self.parts())
+
+    @property
+    def eager_portion_from(self) -> Optional[int]:
+        asked = [n for n in (getattr(p, "eager_portion_from", None) for p in self.parts()) if n is not None]
+        return min(asked) if asked else None
 
 
 def pending_for(norm, pending: Optional[torch.Tensor], dtype: torch.dtype) -> Optional[torch.Tensor]:

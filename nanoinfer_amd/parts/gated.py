@@ -11,6 +11,7 @@ from __future__ import annotations
 
 from typing import Optional
 
+import numpy as np
 import torch
 
 from .. import kernels as K
@@ -74,6 +75,11 @@ class KeyedAttention(WindowAttention):
 
 # ------------------------------------------------------------------ softmax attention over a low-rank latent
 
+# the longest portion of a step from which on a latent attention writes keys and values of every head out for the step
+# (None: never): below it the products over all visible latents cost more than attention over the latents themselves saves
+LATENT_EXPAND_FROM = 256
+
+
 @register_part("mixer", "latent_attention")
 class LatentAttention(Part):
     """Causal softmax attention whose keys and values of every head are projections of one latent ``c`` of ``rank``
@@ -89,7 +95,12 @@ class LatentAttention(Part):
     weights reads the latents that another entry of the order wrote (``LayerRun.writes_cache`` False), with its own
     W_uk, W_uv, queries and window.
 
-    params: hidden_size, num_heads, key_dim, value_dim, q_rank, rank, scale, window (None: every earlier key), eps.
+    Steps whose longest portion has ``expand_from`` tokens or more (and that are not recorded) take the other way:
+    ``k_h`` and ``v_h`` of every latent the step can see are written out once for the step, and attention runs over H
+    heads of ``key_dim`` and ``value_dim`` channels, a fraction of the products where the latent is wider than a head.
+
+    params: hidden_size, num_heads, key_dim, value_dim, q_rank, rank, scale, window (None: every earlier key), eps,
+    expand_from (default ``LATENT_EXPAND_FROM``; None: never; it is never taken where ``rank < key_dim + value_dim``).
     weights: dq [q_rank, d], dq_norm [q_rank], uq [H*dk, q_rank], dkv [rank, d] and dkv_norm [rank] (both or neither),
     uk [H*dk, rank], uv [H*dv, rank], g [H*dv, d], o [d, H*dv]."""
 
@@ -128,6 +139,17 @@ class LatentAttention(Part):
         self.uk = rt.matrix(names["uk"], weights["uk"]).view(self.H, self.dk, self.rank)
         self.uv_t = rt.matrix(names["uv"], weights["uv"]).view(self.H, self.dv, self.rank).transpose(1, 2)
         self.core = PagedSoftmax(self.H, 1, self.rank, self.rank, float(p["scale"]), one_pool=True)
+        # steps with long portions: keys and values of every head are made of the latents the step can see, once,
+        # and attention runs at the heads' own sizes
+        self.expand_from = p.get("expand_from", LATENT_EXPAND_FROM)
+        if self.rank < self.dk + self.dv:      # attention over the latents is then the smaller sum of products already
+            self.expand_from = None
+        if self.expand_from is not None:
+            self.expand_from = max(2, int(self.expand_from))
+        self.eager_portion_from = self.expand_from        # that way reads the step's host lists
+        self.heads = PagedSoftmax(self.H, self.H, self.dk, self.dv, float(p["scale"]))
+        self.uk_rows = self.uk.view(self.H * self.dk, self.rank)
+        self.uv_rows = self.uv_t.transpose(1, 2).view(self.H * self.dv, self.rank)
         K.stream_lib()
 
     def cache_need(self) -> CacheNeed:
@@ -142,6 +164,9 @@ class LatentAttention(Part):
             K.qk_norm_rope_store(proj, ctx.positions, cache.slot_mapping, None, self.dkv_norm, self.eps, None, 1.0, None,
                                  cache.kpool, cache.vpool, 0, col=self.latent_col)
         q = K.linear(K.rmsnorm_cols(proj, 0, self.dq_norm, self.eps, self.rt.dtype), self.w_uq)
+        if self.expand_from is not None and not ctx.recording and ctx.max_q_len >= self.expand_from:
+            y = K.gate_rows(self._over_heads(q, ctx, cache), proj, self.gate_col)
+            return K.linear(y, self.w_o, out_dtype=torch.float32, out=out)
         # the queries as the latents see them, [T, H * rank]: a product per head, read and written in place
         seen = torch.empty(T, H * self.rank, dtype=self.rt.dtype, device=x.device)
         torch.bmm(q.view(T, H, self.dk).transpose(0, 1), self.uk, out=seen.view(T, H, self.rank).transpose(0, 1))
@@ -152,6 +177,31 @@ class LatentAttention(Part):
         K.note_library_call()
         y = K.gate_heads(heads, proj, self.gate_col, self.rt.dtype)
         return K.linear(y, self.w_o, out_dtype=torch.float32, out=out)
+
+
+    def _over_heads(self, q, ctx, cache: LayerCache) -> torch.Tensor:
+        """Attention with keys and values of every head written out: the pages that hold a key some token of the step
+        can see are picked out of the pool, ``k = W_uk c`` and ``v = W_uv c`` are two products over them, laid out as
+        pools of H heads, and the kernels walk them through a block table of their own that holds nothing else.  A
+        tile of queries starts at the tile of 64 keys in which its first token's window starts; the picked pages
+        start there."""
+        ps, window = int(cache.kpool.shape[2]), self.window
+        B, width = cache.block_table.shape
+        pairs, table, at = [], np.full((B, width), -1, dtype=np.int32), 0
+        for b, (n, total) in enumerate(zip(ctx.q_len, ctx.context_len)):
+            first = 0 if window is None else max(total - n - window + 1, 0) // 64 * 64
+            p0, p1 = first // ps, -(-total // ps)
+            pairs.append(np.stack([np.full(p1 - p0, b, dtype=np.int32), np.arange(p0, p1, dtype=np.int32)], axis=1))
+            table[b, p0:p1] = np.arange(at, at + p1 - p0, dtype=np.int32)
+            at += p1 - p0
+        flat = np.concatenate([np.concatenate(pairs).reshape(-1), table.reshape(-1)])
+        upload = getattr(ctx._scratch_owner, "_upload", None)
+        dev = upload(flat) if upload is not None else torch.from_numpy(flat).to(q.device)
+        pairs_dev, table_dev = dev[: 2 * at].view(at, 2), dev[2 * at:].view(B, width)
+        latents = K.gather_pages(cache.kpool, cache.block_table, pairs_dev).view(at * ps, self.rank)
+        keys = K.rows_to_pages(K.linear(latents, self.uk_rows), ps, self.H, self.dk)
+        values = K.rows_to_pages(K.linear(latents, self.uv_rows), ps, self.H, self.dv)
+        return self.heads(q, ctx, keys, values, table_dev, window)
 
 
 # ------------------------------------------------------------------ matrix memory with exponential gates

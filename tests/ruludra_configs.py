@@ -47,6 +47,10 @@ MLP_ONLY = model(56, 83, [(memory(1, 8, 8, 4.0), 50)], eps=1e-3)
 LATENT_SHARED = model(64, 97, [(latent(2, 8, 16, 20, 16, 1.5, mask=9), None), (memory(2, 8, 8, 8.0), None),
                                (latent(4, 12, 8, 12, 16, 1.1, mask=50, kv_from=0), 40),
                                (latent(1, 16, 16, 8, 16, 2.0, mask=3, kv_from=0), None)])
+# latents wider than a head's keys and values together: long portions write the heads' keys and values out for the step
+LATENT_WIDE = model(64, 97, [(latent(3, 8, 8, 24, 32, 1.5, mask=30), None), (memory(2, 8, 8, 8.0), None),
+                             (latent(2, 4, 12, 12, 32, 1.1, mask=70, kv_from=0), 40), (latent(4, 8, 8, 16, 48, 0.9), None),
+                             (latent(1, 16, 8, 8, 32, 2.0, mask=5, kv_from=0), None)])
 # everything together
 MIXED = model(72, 131, [(keyed(6, 2, 16, 0.3, mask=33, temp=(0.5, 16)), 90), (memory(2, 24, 32, 10.0), 44),
                         (latent(3, 16, 24, 40, 32, 1.3, mask=70), None), (keyed(2, 2, 24, 0.2, mask=130), None),
@@ -57,4 +61,4 @@ SHARP = model(64, 97, [(keyed(4, 2, 16, 6.0, mask=19, temp=(0.5, 8)), None), (la
 
 ALL = {"keyed_only": KEYED_ONLY, "keyed_plain": KEYED_PLAIN, "keyed_open": KEYED_OPEN, "latent_only": LATENT_ONLY,
        "latent_open": LATENT_OPEN, "memory_only": MEMORY_ONLY, "memory_wide": MEMORY_WIDE, "mlp_only": MLP_ONLY,
-       "latent_shared": LATENT_SHARED, "mixed": MIXED, "sharp": SHARP}
+       "latent_shared": LATENT_SHARED, "latent_wide": LATENT_WIDE, "mixed": MIXED, "sharp": SHARP}

@@ -502,6 +502,85 @@ def test_matrix_memory_kernels_against_the_plain_recurrence(H, dk, dv, cap, runs
     assert bool(torch.isnan(state[0]).all()) and bool(torch.isfinite(state[1:]).all())
 
 
+# ------------------------------------------------------------------ latents wider than a head: keys and values written out for a step
+
+@pytest.fixture
+def written_out(monkeypatch):
+    """Portions of four tokens or more take the latent attention's other way; counts its calls."""
+    from nanoinfer_amd import kernels as K
+    from nanoinfer_amd.parts import gated
+    calls = []
+    real = K.gather_pages
+    monkeypatch.setattr(gated, "LATENT_EXPAND_FROM", 4)
+    monkeypatch.setattr(K, "gather_pages", lambda *a, **kw: (calls.append(a[2].shape[0]), real(*a, **kw))[1])
+    return calls
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("page_size", [4, 16])
+def test_long_portions_over_written_out_keys_and_values_equal_the_way_over_the_latents(dtype, page_size, written_out):
+    """A model whose latents are wider than a head's keys and values together (read again by two later layers, with a
+    longer and a shorter window, and one layer without a window): the whole prompt, portions on both sides of the
+    threshold in one sequence, and unequal requests in one batch (a long portion beside single tokens and a portion of
+    two, on pages that earlier requests left) against the plain implementation of each request alone."""
+    name = "latent_wide"
+    folder = folder_of(name)
+    vocab = Z.ALL[name]["vocab"]
+    toks = random_tokens(vocab, 150, 31)
+    want = plain(folder, toks)
+    runner = runner_for(folder, dtype, page_size=page_size, max_tokens=320, max_requests=3)
+    assert_close(replay(runner, {"w": toks}, [{"w": len(toks)}])["w"], want, dtype, "whole")
+    assert written_out, "no step took the written-out way"
+    for sizes in ([3, 70, 2, 5, 1], [64, 1, 1, 9], [4, 3]):
+        got = replay(runner, {"p": toks}, [{"p": c} for c in cuts(len(toks), sizes)])["p"]
+        assert_close(got, want, dtype, f"portions of {sizes}")
+    lengths = {"a": 120, "b": 9, "c": 47, "d": 75}
+    requests = {r: random_tokens(vocab, n, 60 + i) for i, (r, n) in enumerate(lengths.items())}
+    steps = [{"a": 40}, {"a": 50, "b": 1, "c": 2}, {"a": 1, "b": 7, "c": 40}, {"c": 1, "a": 29, "b": 1}, {"c": 4}, {"d": 70}, {"d": 5}]
+    got = replay(runner, requests, steps)
+    for r, t in requests.items():
+        assert_close(got[r], plain(folder, t), dtype, f"request {r}")
+    assert not runner.cache.live_requests() and runner.cache.free_pages() == runner.cache.num_pages
+
+
+def test_written_out_keys_and_values_at_a_window_s_edge(written_out):
+    """The sharp model's shape with latents wider than its heads: whether the key at the window's edge is seen decides
+    the output, also where the step's first visible key lies inside a page and inside a tile of 64 keys."""
+    cfg = Z.model(64, 97, [(Z.latent(2, 8, 8, 24, 32, 40.0, mask=23), None), (Z.latent(2, 8, 8, 24, 32, 40.0, mask=66, kv_from=0), None)])
+    import nanoinfer_amd  # noqa: F401
+    from nanoinfer_amd.weights.loader import make_random_model
+    folder = make_random_model(tempfile.mkdtemp(prefix="ruludra-wide-sharp-"), cfg, 5, dtype="bfloat16", matrix_std=0.12)
+    config, w = P.read_model_folder(folder)
+    toks = random_tokens(97, 230, 9)
+    want = torch.from_numpy(P.forward(config, w, list(toks)))
+    runner = runner_for(folder, "float32", page_size=8)
+    assert_close(replay(runner, {"w": toks}, [{"w": len(toks)}])["w"], want, "float32", "whole")
+    got = replay(runner, {"p": toks}, [{"p": c} for c in cuts(len(toks), [100, 7, 90, 33])])["p"]
+    assert_close(got, want, "float32", "portions")
+    assert len(written_out) >= 2 * 5
+    shutil.rmtree(folder, ignore_errors=True)
+
+
+def test_pages_picked_through_a_table_rows_as_pages_and_the_gate_of_rows():
+    from nanoinfer_amd import kernels as K
+    dev = torch.device("cuda")
+    g = torch.Generator().manual_seed(4)
+    for dtype in (torch.float32, torch.bfloat16):
+        pool = torch.randn(9, 1, 4, 10, generator=g).to(dtype).to(dev)
+        table = torch.tensor([[3, -1, 8, 0], [5, 2, -1, -1]], dtype=torch.int32, device=dev)
+        pairs = torch.tensor([[1, 0], [0, 2], [0, 1], [1, 1], [0, 0]], dtype=torch.int32, device=dev)
+        got = K.gather_pages(pool, table, pairs)
+        want = torch.stack([pool[5], pool[8], torch.zeros_like(pool[0]), pool[2], pool[3]])
+        assert torch.equal(got, want)
+        rows = torch.randn(3 * 4, 5 * 6, generator=g).to(dtype).to(dev)
+        assert torch.equal(K.rows_to_pages(rows, 4, 5, 6), rows.view(3, 4, 5, 6).permute(0, 2, 1, 3).contiguous())
+        x = torch.randn(7, 33, generator=g).to(dtype).to(dev)
+        wide = torch.randn(7, 50, generator=g).to(dev)
+        y = K.gate_rows(x, wide, 11)
+        ref = (x.float() * torch.sigmoid(wide[:, 11:44])).to(dtype)
+        assert torch.allclose(y.float(), ref.float(), rtol=1e-2 if dtype == torch.bfloat16 else 1e-6, atol=1e-6)
+
+
 # ------------------------------------------------------------------ the small kernels alone
 
 @pytest.mark.parametrize("T,n", [(1, 50), (7, 352), (70, 33), (3, 4096), (130, 8)])

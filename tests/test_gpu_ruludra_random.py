@@ -65,7 +65,10 @@ def folder_for(cfg, seed):
 
 
 @pytest.mark.parametrize("seed", list(range(1, 15)))
-def test_a_configuration_drawn_at_random(seed):
+def test_a_configuration_drawn_at_random(seed, monkeypatch):
+    if seed % 2:            # portions of sixteen tokens write the heads' keys and values out, where the latents are wide
+        from nanoinfer_amd.parts import gated
+        monkeypatch.setattr(gated, "LATENT_EXPAND_FROM", 16)
     cfg = draw(seed)
     folder = folder_for(cfg, seed)
     config, w = P.read_model_folder(folder)

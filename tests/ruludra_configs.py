@@ -51,6 +51,9 @@ LATENT_SHARED = model(64, 97, [(latent(2, 8, 16, 20, 16, 1.5, mask=9), None), (m
 LATENT_WIDE = model(64, 97, [(latent(3, 8, 8, 24, 32, 1.5, mask=30), None), (memory(2, 8, 8, 8.0), None),
                              (latent(2, 4, 12, 12, 32, 1.1, mask=70, kv_from=0), 40), (latent(4, 8, 8, 16, 48, 0.9), None),
                              (latent(1, 16, 8, 8, 32, 2.0, mask=5, kv_from=0), None)])
+# sizes that are multiples of nothing much: a width of 50, feed-forwards of 37 and 45, a vocabulary of 61
+ODD_SIZES = model(50, 61, [(keyed(2, 1, 12, 0.3, mask=11, temp=(0.4, 3)), 37), (latent(2, 6, 10, 9, 14, 1.2, mask=17), 45),
+                           (memory(1, 12, 9, 5.0), None), (latent(3, 4, 2, 7, 14, 1.4, kv_from=1), None)], bigram=(13, 5, 3))
 # everything together
 MIXED = model(72, 131, [(keyed(6, 2, 16, 0.3, mask=33, temp=(0.5, 16)), 90), (memory(2, 24, 32, 10.0), 44),
                         (latent(3, 16, 24, 40, 32, 1.3, mask=70), None), (keyed(2, 2, 24, 0.2, mask=130), None),
@@ -61,4 +64,4 @@ SHARP = model(64, 97, [(keyed(4, 2, 16, 6.0, mask=19, temp=(0.5, 8)), None), (la
 
 ALL = {"keyed_only": KEYED_ONLY, "keyed_plain": KEYED_PLAIN, "keyed_open": KEYED_OPEN, "latent_only": LATENT_ONLY,
        "latent_open": LATENT_OPEN, "memory_only": MEMORY_ONLY, "memory_wide": MEMORY_WIDE, "mlp_only": MLP_ONLY,
-       "latent_shared": LATENT_SHARED, "latent_wide": LATENT_WIDE, "mixed": MIXED, "sharp": SHARP}
+       "latent_shared": LATENT_SHARED, "latent_wide": LATENT_WIDE, "odd_sizes": ODD_SIZES, "mixed": MIXED, "sharp": SHARP}

@@ -208,7 +208,7 @@ def test_every_mechanism_matters_in_these_models():
 # ------------------------------------------------------------------ the whole design, every schedule
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name", ["mixed", "latent_shared"])
+@pytest.mark.parametrize("name", ["mixed", "latent_shared", "odd_sizes"])
 def test_portions_of_several_sizes_down_to_two_tokens(name, dtype):
     folder = folder_of(name)
     toks = random_tokens(Z.ALL[name]["vocab"], 150, 21)

@@ -140,13 +140,18 @@ class StepContext:
                 return None
             host = self._host
             flat = K.build_q_tiles(host["q_start"], host["q_len"], host["context_len"], tile_tokens)
-            upload = getattr(self._scratch_owner, "_upload", None)
-            if upload is not None:       # through the runner's pinned buffers: the host does not wait for the GPU
-                t = upload(flat).view(-1, 4)
-            else:
-                t = torch.tensor(flat, dtype=torch.int32).view(-1, 4).to(self.device)
+            t = self.upload_ints(flat).view(-1, 4)
             self._q_tiles[tile_tokens] = t
         return t
+
+    def upload_ints(self, flat) -> torch.Tensor:
+        """A list or array of integers as an int32 tensor on the device, for tables a part builds from the host lists
+        of an eager step; through the runner's pinned buffers where there are any, so that the host does not wait for
+        the GPU."""
+        upload = getattr(self._scratch_owner, "_upload", None)
+        if upload is not None:
+            return upload(flat)
+        return torch.as_tensor(np.asarray(flat, dtype=np.int32)).to(self.device)
 
     def workspace(self, n_floats: int) -> torch.Tensor:
         """Float32 scratch that lives until the next request for scratch (one user at a time)."""

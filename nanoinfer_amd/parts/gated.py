@@ -195,8 +195,7 @@ class LatentAttention(Part):
             table[b, p0:p1] = np.arange(at, at + p1 - p0, dtype=np.int32)
             at += p1 - p0
         flat = np.concatenate([np.concatenate(pairs).reshape(-1), table.reshape(-1)])
-        upload = getattr(ctx._scratch_owner, "_upload", None)
-        dev = upload(flat) if upload is not None else torch.from_numpy(flat).to(q.device)
+        dev = ctx.upload_ints(flat)
         pairs_dev, table_dev = dev[: 2 * at].view(at, 2), dev[2 * at:].view(B, width)
         latents = K.gather_pages(cache.kpool, cache.block_table, pairs_dev).view(at * ps, self.rank)
         keys = K.rows_to_pages(K.linear(latents, self.uk_rows), ps, self.H, self.dk)

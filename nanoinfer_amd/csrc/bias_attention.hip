@@ -14,6 +14,10 @@
 // tiles from the one in which the window of the tile's first token starts (`KeyWalk`).  `out_scale` multiplies the
 // normalised output (a mixer that is one of several side by side has a weight of its own).
 //
+// A sink (`sink`, float32 [heads], or null) is one more term exp(sink[head]) in a row's denominator, with no key and
+// no value: the weights of a row then sum to less than one.  It counts once a row, whatever the number of runs: the
+// kernels add it when a row is finished (a row in runs: when the runs are merged).
+//
 // One workgroup of four wavefronts takes a tile of consecutive tokens of one sequence and (a chunk of)
 // the query heads of one kv head: 16 rows of (token, head), four a wavefront.  64 keys and values at a
 // time are staged in LDS as float32 for the whole workgroup; a lane owns one key of the 64 for the
@@ -72,38 +76,67 @@ __global__ void kv_store_kernel(const T* __restrict__ qkv, int row_stride, int k
 }
 
 // The same for projections that still want their norm and rotation, all of it in float32:
-//   q <- rotate(rmsnorm(q) * wq), k <- rotate(rmsnorm(k) * wk)      the norms run over the WHOLE projection of a token
-//   (all heads at once; a null weight: no norm), the rotation turns channel c < rot/2 of every head together with
-//   channel c + rot/2 by the angle position * freq[c], cos and sin times `amplitude` (a null freq: no rotation);
-//   the channels from `rot` on pass as they are.
-// proj float32 [T, row_stride] holds q [H * dk] | k [G * dk] | v [G * dv] (`v_from_k`: no v; the values are the keys as
-// projected, before their norm, and dv = dk); q goes to q_out [T, H * dk] in the compute
+//   q <- rotate(rmsnorm(q) * wq), k <- rotate(rmsnorm(k) * wk)
+//   The norms (a null weight: no norm) run over the WHOLE projection of a token, all heads at once, weights [H * dq]
+//   and [G * dk]; or, `per_head`, over every head on its own with one weight [dq] (or [k_normed]) shared by the heads.
+//   Of a key head only the first `k_normed` channels are normed (whole-projection norms: all of them); the others
+//   pass as projected.
+//   The rotation (a null freq: none) turns `rot` channels of every head, from channel `rot_at_q` (queries) or
+//   `rot_at_k` (keys) on, by the angles position * freq[p], cos and sin times `amplitude`: channel c of them with
+//   channel c + rot/2, or, `adjacent`, channel 2p with channel 2p + 1.  The other channels pass as they are.
+// proj float32 [T, row_stride] holds q [H * dq] | k [G * dk] | v [G * dv] (`v_from_k`: no v; the values are the keys as
+// projected, before their norm, and dv = dk); q goes to q_out [T, H * dq] in the compute
 // type, k and v into their page slots.  A token is taken by gridDim.y workgroups, each with its share of the elements
-// (and the sums of squares over the whole projections, which every one of them works out): one for steps of many
+// (and the sums of squares, which every one of them works out): one for steps of many
 // tokens; a step of few tokens, where one workgroup a token would walk its row alone, spreads the row.
-#define ROT_PAIRS 128          // rotated pairs of a head at most: heads of up to 256 channels
+#define ROT_PAIRS 128          // rotated pairs of a head at most: heads of up to 256 rotated channels
+#define NORM_HEADS 1024        // heads of queries and keys together that are normed one by one, at most
+
+struct QkForm {
+    int H, G, dq, dk, dv, k_normed, rot, rot_at_q, rot_at_k;
+    bool v_from_k, per_head, adjacent;
+};
 
 template <typename T>
 __global__ void __launch_bounds__(256)
 qk_norm_rope_store_kernel(const float* __restrict__ proj, int row_stride, const int32_t* __restrict__ positions,
                           const int32_t* __restrict__ slot_mapping, const float* __restrict__ wq, const float* __restrict__ wk,
-                          float eps, const float* __restrict__ freq, int rot, float amplitude, T* __restrict__ q_out,
-                          T* __restrict__ kpool, T* __restrict__ vpool, int H, int G, int dk, int dv, int page_size, bool v_from_k) {
+                          float eps, const float* __restrict__ freq, float amplitude, T* __restrict__ q_out,
+                          T* __restrict__ kpool, T* __restrict__ vpool, int page_size, QkForm f) {
     __shared__ float scratch[8];
     __shared__ float cos_of[ROT_PAIRS], sin_of[ROT_PAIRS];     // the token's angles, worked out once for all heads
+    __shared__ float head_r[NORM_HEADS];                       // per_head: 1 / rms of every query head, then of every key head
     const int t = blockIdx.x, tid = threadIdx.x;
     const float* row = proj + static_cast<size_t>(t) * row_stride;
-    const int nq = H * dk, nk = G * dk;
+    const int H = f.H, G = f.G, dq = f.dq, dk = f.dk, dv = f.dv, rot = f.rot;
+    const int nq = H * dq, nk = G * dk;
     float rq = 1.f, rk = 1.f;
-    if (wq) {
-        float ss = 0.f;
-        for (int i = tid; i < nq; i += blockDim.x) ss += row[i] * row[i];
-        rq = 1.0f / sqrtf(block_sum(ss, scratch) / static_cast<float>(nq) + eps);
-    }
-    if (wk) {
-        float ss = 0.f;
-        for (int i = tid; i < nk; i += blockDim.x) ss += row[nq + i] * row[nq + i];
-        rk = 1.0f / sqrtf(block_sum(ss, scratch) / static_cast<float>(nk) + eps);
+    if (f.per_head) {
+        // a head a wavefront at a time: its lanes walk the head's normed channels
+        const int lane = tid & (WAVE - 1), wave = tid / WAVE, waves = blockDim.x / WAVE;
+        for (int hd = wave; hd < H + G; hd += waves) {
+            const bool is_q = hd < H;
+            const float* w = is_q ? wq : wk;
+            if (!w) continue;                                  // the same for the whole wavefront
+            const float* src = is_q ? row + hd * dq : row + nq + (hd - H) * dk;
+            const int n = is_q ? dq : f.k_normed;
+            float ss = 0.f;
+            for (int c = lane; c < n; c += WAVE) ss += src[c] * src[c];
+            ss = wave_sum(ss);
+            if (lane == 0) head_r[hd] = 1.0f / sqrtf(ss / static_cast<float>(n) + eps);
+        }
+        __syncthreads();
+    } else {
+        if (wq) {
+            float ss = 0.f;
+            for (int i = tid; i < nq; i += blockDim.x) ss += row[i] * row[i];
+            rq = 1.0f / sqrtf(block_sum(ss, scratch) / static_cast<float>(nq) + eps);
+        }
+        if (wk) {
+            float ss = 0.f;
+            for (int i = tid; i < nk; i += blockDim.x) ss += row[nq + i] * row[nq + i];
+            rk = 1.0f / sqrtf(block_sum(ss, scratch) / static_cast<float>(nk) + eps);
+        }
     }
     const float pos = static_cast<float>(positions[t]);
     const int half = rot / 2;
@@ -125,25 +158,33 @@ qk_norm_rope_store_kernel(const float* __restrict__ proj, int row_stride, const 
         const int j = is_q ? i : i - nq;                 // index inside the projection
         const float* src = is_q ? row : row + nq;
         const float* w = is_q ? wq : wk;
-        const float r = is_q ? rq : rk;
-        const int c = j % dk;
-        float v = src[j] * r * (w ? w[j] : 1.f);
-        if (freq && c < rot) {
-            const int jp = c < half ? j + half : j - half;
-            const float other = src[jp] * r * (w ? w[jp] : 1.f);
-            const int p = c < half ? c : c - half;
+        const int size = is_q ? dq : dk;
+        const int hd = j / size, c = j - hd * size;
+        const int normed = !w ? 0 : (is_q ? size : f.k_normed);       // leading channels of the head that are normed
+        const float r = f.per_head ? (w ? head_r[is_q ? hd : H + hd] : 1.f) : (is_q ? rq : rk);
+        // the element at channel cc of this head, after its norm
+        auto normed_at = [&](int cc) -> float {
+            const float x = src[hd * size + cc];
+            return cc < normed ? x * r * w[f.per_head ? cc : hd * size + cc] : x;
+        };
+        float v = normed_at(c);
+        const int cr = c - (is_q ? f.rot_at_q : f.rot_at_k);           // index among the rotated channels
+        if (freq && cr >= 0 && cr < rot) {
+            const bool first = f.adjacent ? !(cr & 1) : cr < half;
+            const int partner = f.adjacent ? (cr ^ 1) : (first ? cr + half : cr - half);
+            const int p = f.adjacent ? (cr >> 1) : (first ? cr : cr - half);
+            const float other = normed_at(c - cr + partner);
             const float cs = cos_of[p], sn = sin_of[p];
-            v = c < half ? v * cs - other * sn : v * cs + other * sn;
+            v = first ? v * cs - other * sn : v * cs + other * sn;
         }
         if (is_q) {
             st(q_out + static_cast<size_t>(t) * nq + j, v);
         } else if (slot >= 0) {
-            const int g = j / dk;
-            st(kpool + ((static_cast<size_t>(page) * G + g) * page_size + in_page) * dk + c, v);
+            st(kpool + ((static_cast<size_t>(page) * G + hd) * page_size + in_page) * dk + c, v);
         }
     }
     if (slot >= 0) {
-        const float* vsrc = v_from_k ? row + nq : row + nq + nk;      // the values may be the keys as projected, before their norm
+        const float* vsrc = f.v_from_k ? row + nq : row + nq + nk;      // the values may be the keys as projected, before their norm
         const int vper = (G * dv + slices - 1) / slices;
         for (int i = slice * vper + tid; i < min(G * dv, (slice + 1) * vper); i += blockDim.x) {
             const int g = i / dv, c = i % dv;
@@ -152,24 +193,33 @@ qk_norm_rope_store_kernel(const float* __restrict__ proj, int row_stride, const 
     }
 }
 
+// `per_head`, `adjacent`, `dq`, `k_normed`, `rot_at_q`, `rot_at_k`: see the kernel.  G may be 0 (queries alone).
 NI_EXPORT int ni_qk_norm_rope_store(const void* proj, int row_stride, const void* positions, const void* slot_mapping,
                                     const void* wq, const void* wk, float eps, const void* freq, int rot, float amplitude,
-                                    void* q_out, void* kpool, void* vpool, int T, int H, int G, int dk, int dv, int page_size,
-                                    int v_from_k, int dtype, hipStream_t stream) {
+                                    void* q_out, void* kpool, void* vpool, int T, int H, int G, int dq, int dk, int dv, int page_size,
+                                    int v_from_k, int per_head, int k_normed, int rot_at_q, int rot_at_k, int adjacent,
+                                    int dtype, hipStream_t stream) {
     if (T <= 0) return 0;
-    if (rot < 0 || rot > dk || rot % 2 || rot > 2 * ROT_PAIRS || row_stride < H * dk + G * dk + (v_from_k ? 0 : G * dv)) return -1;
+    if (H < 0 || G < 0 || dq < 0 || dk < 0 || dv < 0 || (H > 0 && dq < 1) || (G > 0 && dk < 1)) return -1;
+    if (rot < 0 || rot % 2 || rot > 2 * ROT_PAIRS || rot_at_q < 0 || rot_at_k < 0) return -1;
+    if (freq && ((H > 0 && rot_at_q + rot > dq) || (G > 0 && rot_at_k + rot > dk))) return -1;
+    if (row_stride < H * dq + G * dk + (v_from_k ? 0 : G * dv)) return -1;
     if (v_from_k && dv != dk) return -1;
+    if (k_normed < 0 || k_normed > dk || (!per_head && wk && k_normed != dk)) return -1;
+    if (per_head && H + G > NORM_HEADS) return -1;
+    if ((H > 0 && !q_out) || (G > 0 && slot_mapping && (!kpool || (dv > 0 && !vpool)))) return -1;
+    const QkForm f{H, G, dq, dk, dv, k_normed, freq ? rot : 0, rot_at_q, rot_at_k, v_from_k != 0, per_head != 0, adjacent != 0};
     // few tokens: a row's elements over several workgroups, one pass of 256 threads each
-    const int slices = T >= 64 ? 1 : std::max(1, std::min(16, ((H + G) * dk + 255) / 256));
+    const int slices = T >= 64 ? 1 : std::max(1, std::min(16, (H * dq + G * dk + 255) / 256));
     const dim3 grid(T, slices);
     if (dtype == 0)
         qk_norm_rope_store_kernel<float><<<grid, 256, 0, stream>>>((const float*)proj, row_stride, (const int32_t*)positions,
-            (const int32_t*)slot_mapping, (const float*)wq, (const float*)wk, eps, (const float*)freq, rot, amplitude,
-            (float*)q_out, (float*)kpool, (float*)vpool, H, G, dk, dv, page_size, v_from_k != 0);
+            (const int32_t*)slot_mapping, (const float*)wq, (const float*)wk, eps, (const float*)freq, amplitude,
+            (float*)q_out, (float*)kpool, (float*)vpool, page_size, f);
     else
         qk_norm_rope_store_kernel<bf16_t><<<grid, 256, 0, stream>>>((const float*)proj, row_stride, (const int32_t*)positions,
-            (const int32_t*)slot_mapping, (const float*)wq, (const float*)wk, eps, (const float*)freq, rot, amplitude,
-            (bf16_t*)q_out, (bf16_t*)kpool, (bf16_t*)vpool, H, G, dk, dv, page_size, v_from_k != 0);
+            (const int32_t*)slot_mapping, (const float*)wq, (const float*)wk, eps, (const float*)freq, amplitude,
+            (bf16_t*)q_out, (bf16_t*)kpool, (bf16_t*)vpool, page_size, f);
     return NI_LAUNCH_RESULT();
 }
 
@@ -298,7 +348,7 @@ bias_attention_kernel(const T* __restrict__ qkv, int row_stride, const T* __rest
                       const int32_t* __restrict__ positions, const float* __restrict__ bias, int distances, T* __restrict__ out, int H, int G, int dk, int dv,
                       int page_size, float scale, float temp_coef, int temp_every, int heads_per_chunk, int n_runs,
                       float* __restrict__ partial, bool k_pieces, bool v_pieces, int dkp, int window, int keep_first,
-                      float out_scale) {
+                      float out_scale, const float* __restrict__ sink) {
     extern __shared__ __attribute__((aligned(16))) float lds[];
     // a lane reads its key's row: the stride is the row plus four floats where rows are whole 16-byte pieces (read
     // as such), plus one otherwise; both spread the lanes over the banks
@@ -434,7 +484,11 @@ bias_attention_kernel(const T* __restrict__ qkv, int row_stride, const T* __rest
             continue;
         }
         T* orow = out + static_cast<size_t>(first_row + r / heads_here) * (H * dv) + head[rr] * dv;
-        const float inv = out_scale / l[rr];
+        float inv = out_scale / l[rr];
+        if (sink) {             // one more term in the denominator: with M = max(m, sink), l e^(m - M) + e^(sink - M)
+            const float sk = sink[head[rr]], M = fmaxf(m[rr], sk), w = expf(m[rr] - M);
+            inv = out_scale * w / (l[rr] * w + expf(sk - M));
+        }
 #pragma unroll
         for (int cc = 0; cc < MAX_VCHUNKS; ++cc) {
             const int c = lane + cc * WAVE;
@@ -476,7 +530,7 @@ bias_attention_mfma_kernel(const T* __restrict__ qkv, int row_stride, const T* _
                            const int32_t* __restrict__ positions, const float* __restrict__ bias, int distances,
                            T* __restrict__ out, int H, int G, int dk, int dv, int page_size, float scale, float temp_coef,
                            int temp_every, int heads_per_chunk, bool k_pieces, bool v_pieces, int window, int keep_first,
-                           float out_scale) {
+                           float out_scale, const float* __restrict__ sink) {
     extern __shared__ __attribute__((aligned(16))) float lds[];
     const int dkp = dk + 4, dvp = dv + 4;         // strides that spread the sixteen rows of a read over the banks
     float* Qs = lds;                              // [MROWS][dkp]
@@ -585,7 +639,11 @@ bias_attention_mfma_kernel(const T* __restrict__ qkv, int row_stride, const T* _
     }
     if (!valid) return;
     T* orow = out + static_cast<size_t>(first_row + row / heads_here) * (H * dv) + head * dv + 4 * kg;
-    const float inv = out_scale / l;
+    float inv = out_scale / l;
+    if (sink) {                 // one more term in the denominator: with M = max(m, sink), l e^(m - M) + e^(sink - M)
+        const float sk = sink[head], M = fmaxf(m, sk), w = expf(m - M);
+        inv = out_scale * w / (l * w + expf(sk - M));
+    }
 #pragma unroll
     for (int db = 0; db < MAX_VCHUNKS * 4; ++db) {
         if (db < dvb) {
@@ -595,12 +653,13 @@ bias_attention_mfma_kernel(const T* __restrict__ qkv, int row_stride, const T* _
     }
 }
 
-// out[row, :] = sum_r acc_r e^(m_r - M) / sum_r l_r e^(m_r - M) over the runs of a row (an empty run has l = 0).
+// out[row, :] = sum_r acc_r e^(m_r - M) / (sum_r l_r e^(m_r - M) + e^(sink - M)) over the runs of a row (an empty run
+// has l = 0; no sink: no such term; M is the maximum over the runs and the sink).
 // One wavefront a row; lane r takes run r's maximum and sum (n_runs <= 64), the weights e^(m_r - M) go through LDS,
 // and the sums over the runs then read nothing that depends on an earlier read.
 template <typename T>
 __global__ void __launch_bounds__(WAVE) merge_runs_kernel(const float* __restrict__ partial, T* __restrict__ out, int n_runs, int dv,
-                                                          float out_scale) {
+                                                          float out_scale, const float* __restrict__ sink, int H) {
     __shared__ float weight[WAVE];
     const size_t row = blockIdx.x;
     const float* p = partial + row * n_runs * (dv + 2);
@@ -611,9 +670,11 @@ __global__ void __launch_bounds__(WAVE) merge_runs_kernel(const float* __restric
         l = p[lane * (dv + 2) + 1];
     }
     if (!(l > 0.f)) m = -INFINITY;
-    const float M = wave_max(m);
+    float M = wave_max(m);
+    const float sk = sink ? sink[row % H] : -INFINITY;        // rows are (token, head); the sink counts once, here
+    M = fmaxf(M, sk);
     const float w = l > 0.f ? expf(m - M) : 0.f;
-    const float L = wave_sum(l * w);
+    const float L = wave_sum(l * w) + (sink ? expf(sk - M) : 0.f);
     weight[lane] = w;
     __syncthreads();
     for (int c = lane; c < dv; c += WAVE) {
@@ -644,7 +705,7 @@ NI_EXPORT int ni_bias_attention(const void* qkv, int row_stride, const void* kpo
                                 int table_width, const void* tiles, int n_tiles, const void* positions, const void* bias, int distances, void* out,
                                 int H, int G, int dk, int dv, int page_size, float scale, float temp_coef, int temp_every,
                                 int heads_per_chunk, int n_runs, void* partial, int n_rows, int waves, int window, int keep_first,
-                                float out_scale, int dtype, hipStream_t stream) {
+                                float out_scale, const void* sink, int dtype, hipStream_t stream) {
     if (n_tiles <= 0) return 0;
     if (window < 0 || keep_first < 0) return -1;
     if (dv > MAX_VCHUNKS * WAVE || H % G || heads_per_chunk < 1 || heads_per_chunk > ROWS) return -1;
@@ -668,8 +729,10 @@ NI_EXPORT int ni_bias_attention(const void* qkv, int row_stride, const void* kpo
         bias_attention_kernel<float><<<grid, waves * WAVE, lds, stream>>>(
             (const float*)qkv, row_stride, (const float*)kpool, (const float*)vpool, (const int32_t*)block_table, table_width,
             (const int32_t*)tiles, (const int32_t*)positions, (const float*)bias, distances, (float*)out, H, G, dk, dv, page_size, scale, temp_coef,
-            temp_every, heads_per_chunk, n_runs, (float*)partial, k_pieces, v_pieces, dkp, window, keep_first, out_scale);
-        if (partial) merge_runs_kernel<float><<<n_rows * H, 64, 0, stream>>>((const float*)partial, (float*)out, n_runs, dv, out_scale);
+            temp_every, heads_per_chunk, n_runs, (float*)partial, k_pieces, v_pieces, dkp, window, keep_first, out_scale,
+            (const float*)sink);
+        if (partial) merge_runs_kernel<float><<<n_rows * H, 64, 0, stream>>>((const float*)partial, (float*)out, n_runs, dv, out_scale,
+                                                                             (const float*)sink, H);
     } else {
         static size_t allowed = 48 * 1024;
         if (lds > allowed && (allowed = lds))
@@ -678,8 +741,10 @@ NI_EXPORT int ni_bias_attention(const void* qkv, int row_stride, const void* kpo
         bias_attention_kernel<bf16_t><<<grid, waves * WAVE, lds, stream>>>(
             (const bf16_t*)qkv, row_stride, (const bf16_t*)kpool, (const bf16_t*)vpool, (const int32_t*)block_table, table_width,
             (const int32_t*)tiles, (const int32_t*)positions, (const float*)bias, distances, (bf16_t*)out, H, G, dk, dv, page_size, scale, temp_coef,
-            temp_every, heads_per_chunk, n_runs, (float*)partial, k_pieces, v_pieces, dkp, window, keep_first, out_scale);
-        if (partial) merge_runs_kernel<bf16_t><<<n_rows * H, 64, 0, stream>>>((const float*)partial, (bf16_t*)out, n_runs, dv, out_scale);
+            temp_every, heads_per_chunk, n_runs, (float*)partial, k_pieces, v_pieces, dkp, window, keep_first, out_scale,
+            (const float*)sink);
+        if (partial) merge_runs_kernel<bf16_t><<<n_rows * H, 64, 0, stream>>>((const float*)partial, (bf16_t*)out, n_runs, dv, out_scale,
+                                                                              (const float*)sink, H);
     }
     return NI_LAUNCH_RESULT();
 }
@@ -701,7 +766,7 @@ NI_EXPORT int ni_bias_attention_mfma(const void* qkv, int row_stride, const void
                                      int table_width, const void* tiles, int n_tiles, const void* positions, const void* bias,
                                      int distances, void* out, int H, int G, int dk, int dv, int page_size, float scale,
                                      float temp_coef, int temp_every, int heads_per_chunk, int window, int keep_first,
-                                     float out_scale, int dtype, hipStream_t stream) {
+                                     float out_scale, const void* sink, int dtype, hipStream_t stream) {
     if (n_tiles <= 0) return 0;
     if (window < 0 || keep_first < 0) return -1;
     const bool one_pool = kpool == vpool && dk == dv;
@@ -721,7 +786,7 @@ NI_EXPORT int ni_bias_attention_mfma(const void* qkv, int row_stride, const void
         bias_attention_mfma_kernel<float><<<grid, WAVES * WAVE, lds, stream>>>(
             (const float*)qkv, row_stride, (const float*)kpool, (const float*)vpool, (const int32_t*)block_table, table_width,
             (const int32_t*)tiles, (const int32_t*)positions, (const float*)bias, distances, (float*)out, H, G, dk, dv, page_size,
-            scale, temp_coef, temp_every, heads_per_chunk, k_pieces, v_pieces, window, keep_first, out_scale);
+            scale, temp_coef, temp_every, heads_per_chunk, k_pieces, v_pieces, window, keep_first, out_scale, (const float*)sink);
     } else {
         static size_t allowed = 48 * 1024;
         if (lds > allowed && (allowed = lds))
@@ -730,7 +795,7 @@ NI_EXPORT int ni_bias_attention_mfma(const void* qkv, int row_stride, const void
         bias_attention_mfma_kernel<bf16_t><<<grid, WAVES * WAVE, lds, stream>>>(
             (const bf16_t*)qkv, row_stride, (const bf16_t*)kpool, (const bf16_t*)vpool, (const int32_t*)block_table, table_width,
             (const int32_t*)tiles, (const int32_t*)positions, (const float*)bias, distances, (bf16_t*)out, H, G, dk, dv, page_size,
-            scale, temp_coef, temp_every, heads_per_chunk, k_pieces, v_pieces, window, keep_first, out_scale);
+            scale, temp_coef, temp_every, heads_per_chunk, k_pieces, v_pieces, window, keep_first, out_scale, (const float*)sink);
     }
     return NI_LAUNCH_RESULT();
 }

@@ -241,6 +241,50 @@ NI_EXPORT int ni_add_rmsnormed(void* h, const void* y, const void* w, int T, int
     return NI_LAUNCH_RESULT();
 }
 
+// ---------------------------------------------------------------- the stream behind a norm: h = rmsnorm(alpha h + sum of addends) * w
+// The stream itself takes the normed sum (a block whose norm stands behind the sum); x, if given, is the same in the
+// compute type for the products that read it next.  addends float32 [n_addends][T][d], summed in their order and then
+// added to alpha * h; all of it float32.  A thread reads in the second pass what it wrote itself in the first.
+template <typename X>
+__global__ void post_norm_kernel(float* __restrict__ h, const float* __restrict__ addends, int n_addends, size_t addend_stride,
+                                 float alpha, const float* __restrict__ w, float eps, X* __restrict__ x, int d) {
+    __shared__ float scratch[16];
+    const size_t base = static_cast<size_t>(blockIdx.x) * d;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < d; i += blockDim.x) {
+        float v = alpha * h[base + i];
+        if (n_addends > 0) {
+            float a = addends[base + i];
+            for (int s = 1; s < n_addends; ++s) a += addends[s * addend_stride + base + i];
+            v += a;
+        }
+        h[base + i] = v;
+        ss += v * v;
+    }
+    ss = block_sum(ss, scratch);
+    const float inv = 1.0f / sqrtf(ss / static_cast<float>(d) + eps);
+    for (int i = threadIdx.x; i < d; i += blockDim.x) {
+        const float v = (h[base + i] * inv) * w[i];
+        h[base + i] = v;
+        if (x) st(x + base + i, v);
+    }
+}
+
+NI_EXPORT int ni_post_norm(void* h, const void* addends, int n_addends, float alpha, const void* w, float eps, void* x, int x_dtype,
+                           int T, int d, hipStream_t stream) {
+    if (T <= 0 || d <= 0) return 0;
+    if (n_addends < 0 || (n_addends > 0 && !addends)) return -1;
+    const int threads = d <= 256 ? 64 : d <= 1024 ? 256 : 512;
+    const size_t stride = static_cast<size_t>(T) * d;
+    if (x_dtype == 0)
+        post_norm_kernel<float><<<T, threads, 0, stream>>>((float*)h, (const float*)addends, n_addends, stride, alpha, (const float*)w, eps,
+                                                           (float*)x, d);
+    else
+        post_norm_kernel<bf16_t><<<T, threads, 0, stream>>>((float*)h, (const float*)addends, n_addends, stride, alpha, (const float*)w, eps,
+                                                            (bf16_t*)x, d);
+    return NI_LAUNCH_RESULT();
+}
+
 // ---------------------------------------------------------------- y = x / sqrt(mean(x^2) + eps) * w over columns of wider rows
 // x: n columns of float32 rows of stride `stride` (a product's accumulators); y [T, n] in the type T
 template <typename T>
@@ -358,26 +402,27 @@ NI_EXPORT int ni_scale(void* x, float s, size_t n, hipStream_t stream) {
 }
 
 // ---------------------------------------------------------------- read-outs head by head times a gate
-//   y[t, h * dv + c] = o[h][t][c] * sigmoid(g[t, h * dv + c])      o float32 [H][T][dv], g float32 rows of stride g_stride
+//   y[t, h * dv + c] = o[h][t][c] * sigmoid(g[t, (h * dv + c) / per])      o float32 [H][T][dv], g float32 rows of stride
+//   g_stride; per = 1: a gate a channel, per = dv: a gate a head
 template <typename T>
 __global__ void gate_heads_kernel(const float* __restrict__ o, const float* __restrict__ g, int g_stride, T* __restrict__ y,
-                                  int Tn, int H, int dv, size_t total) {
+                                  int Tn, int H, int dv, int per, size_t total) {
     const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (i >= total) return;
     const int c = static_cast<int>(i % dv), h = static_cast<int>((i / dv) % H);
     const size_t t = i / (static_cast<size_t>(dv) * H);
-    const float gate = 1.0f / (1.0f + expf(-g[t * g_stride + h * dv + c]));
+    const float gate = 1.0f / (1.0f + expf(-g[t * g_stride + (h * dv + c) / per]));
     st(y + i, o[(static_cast<size_t>(h) * Tn + t) * dv + c] * gate);
 }
 
-NI_EXPORT int ni_gate_heads(const void* o, const void* g, int g_stride, void* y, int T, int H, int dv, int dtype, hipStream_t stream) {
+NI_EXPORT int ni_gate_heads(const void* o, const void* g, int g_stride, void* y, int T, int H, int dv, int per, int dtype, hipStream_t stream) {
     const size_t total = static_cast<size_t>(T) * H * dv;
     if (total == 0) return 0;
-    if (g_stride < H * dv) return -1;
+    if (per < 1 || g_stride < (H * dv + per - 1) / per) return -1;
     if (dtype == 0)
-        gate_heads_kernel<float><<<blocks_of(total, 256), 256, 0, stream>>>((const float*)o, (const float*)g, g_stride, (float*)y, T, H, dv, total);
+        gate_heads_kernel<float><<<blocks_of(total, 256), 256, 0, stream>>>((const float*)o, (const float*)g, g_stride, (float*)y, T, H, dv, per, total);
     else
-        gate_heads_kernel<bf16_t><<<blocks_of(total, 256), 256, 0, stream>>>((const float*)o, (const float*)g, g_stride, (bf16_t*)y, T, H, dv, total);
+        gate_heads_kernel<bf16_t><<<blocks_of(total, 256), 256, 0, stream>>>((const float*)o, (const float*)g, g_stride, (bf16_t*)y, T, H, dv, per, total);
     return NI_LAUNCH_RESULT();
 }
 
@@ -405,26 +450,27 @@ NI_EXPORT int ni_heads_apart(const void* x, int x_stride, void* y, int T, int H,
 }
 
 // ---------------------------------------------------------------- rows times the sigmoid of a gate
-//   y[t, j] = x[t, j] * sigmoid(g[t, j])      x [T, n] in the compute type, g float32 rows of stride g_stride
+//   y[t, j] = x[t, j] * sigmoid(g[t, j / per])      x [T, n] in the compute type, g float32 rows of stride g_stride;
+//   per = 1: a gate a channel, per = a head's channels: a gate a head
 template <typename T>
 __global__ void gate_rows_kernel(const T* __restrict__ x, const float* __restrict__ g, int g_stride, T* __restrict__ y, int n,
-                                 size_t total) {
+                                 int per, size_t total) {
     const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (i >= total) return;
     const size_t t = i / n;
     const int j = static_cast<int>(i % n);
-    const float gate = 1.0f / (1.0f + expf(-g[t * g_stride + j]));
+    const float gate = 1.0f / (1.0f + expf(-g[t * g_stride + j / per]));
     st(y + i, ld(x + i) * gate);
 }
 
-NI_EXPORT int ni_gate_rows(const void* x, const void* g, int g_stride, void* y, int T, int n, int dtype, hipStream_t stream) {
+NI_EXPORT int ni_gate_rows(const void* x, const void* g, int g_stride, void* y, int T, int n, int per, int dtype, hipStream_t stream) {
     const size_t total = static_cast<size_t>(T) * n;
     if (total == 0) return 0;
-    if (g_stride < n) return -1;
+    if (per < 1 || g_stride < (n + per - 1) / per) return -1;
     if (dtype == 0)
-        gate_rows_kernel<float><<<blocks_of(total, 256), 256, 0, stream>>>((const float*)x, (const float*)g, g_stride, (float*)y, n, total);
+        gate_rows_kernel<float><<<blocks_of(total, 256), 256, 0, stream>>>((const float*)x, (const float*)g, g_stride, (float*)y, n, per, total);
     else
-        gate_rows_kernel<bf16_t><<<blocks_of(total, 256), 256, 0, stream>>>((const bf16_t*)x, (const float*)g, g_stride, (bf16_t*)y, n, total);
+        gate_rows_kernel<bf16_t><<<blocks_of(total, 256), 256, 0, stream>>>((const bf16_t*)x, (const float*)g, g_stride, (bf16_t*)y, n, per, total);
     return NI_LAUNCH_RESULT();
 }
 
@@ -478,33 +524,47 @@ NI_EXPORT int ni_rows_to_pages(const void* x, void* y, int n_pages, int page, in
 }
 
 // ---------------------------------------------------------------- the router's choice
-// z float32 [T, E]: the `top` largest logits of a row (the lower index on equal logits) and their weights:
-// the softmax among the chosen (`over_all` 0) or the softmax over all E experts, not renormalised (`over_all` 1).
-// With `n_groups` > 1 the experts form that many equal groups of neighbours; a group counts as much as its
-// largest logit, and only experts of the `keep` best groups (the lower index on equal ones) can be chosen.
+// z float32 [T, E]: the `top` experts of a row with the largest scores (the lower index on equal scores) and their weights.
+// `scoring` says what an expert's value is and how the chosen ones are weighed:
+//   0  the logit; weights: the softmax among the chosen
+//   1  the logit; weights: the softmax over all E experts, not renormalised
+//   2  sigmoid(logit); weights: the values themselves, not renormalised
+// every weight times `route_scale`.  An expert is chosen by its value plus `correction[e]` (float32 [E]; null: the value
+// alone); the weights never see the correction.
+// With `n_groups` > 1 the experts form that many equal groups of neighbours; a group counts as much as the sum of its
+// `group_top` largest scores (1: its largest score), and only experts of the `keep` best groups (the lower index on
+// equal ones) can be chosen: the others' scores count as minus infinity.
 // chosen int32 [T, top], mix float32 [T, top], and (if asked for) the same as a row over all experts, zero where
 // an expert was not chosen.
-// One wavefront a row: a lane keeps the logits of experts lane, lane + 64, ...; each of the `top` rounds finds the
-// largest logit not yet taken (the lowest index among equal ones) by two butterflies over the lanes.
+// One wavefront a row: a lane keeps the scores of experts lane, lane + 64, ...; each round finds the
+// largest score not yet taken (the lowest index among equal ones) by two butterflies over the lanes.
+#define NO_EXPERT 0x7fffffff
+
+__device__ __forceinline__ int lowest_of(int cand) {
+#pragma unroll
+    for (int off = WAVE / 2; off > 0; off >>= 1) cand = min(cand, __shfl_xor(cand, off, WAVE));
+    return cand;
+}
+
 template <int SLOTS>
-__global__ void route_top_kernel(const float* __restrict__ z, int32_t* __restrict__ chosen, float* __restrict__ mix,
-                                 float* __restrict__ mix_all, int T, int E, int top, int over_all, int n_groups, int keep) {
+__global__ void route_top_kernel(const float* __restrict__ z, const float* __restrict__ correction, int32_t* __restrict__ chosen,
+                                 float* __restrict__ mix, float* __restrict__ mix_all, int T, int E, int top, int scoring,
+                                 int n_groups, int keep, int group_top, float route_scale) {
     const int t = blockIdx.x, lane = threadIdx.x;
     const float* row = z + static_cast<size_t>(t) * E;
     int32_t* c = chosen + static_cast<size_t>(t) * top;
     float* m = mix + static_cast<size_t>(t) * top;
     // the row once, into registers: slot j of a lane is expert lane + 64 j (every round below would else wait for memory
-    // again); a logit that is no number is never preferred
-    float vals[SLOTS];
+    // again); a logit that is no number is never preferred.  vals: what chooses; raw: what weighs
+    float vals[SLOTS], raw[SLOTS];
 #pragma unroll
     for (int j = 0; j < SLOTS; ++j) {
         const int e = lane + j * WAVE;
         float ze = e < E ? row[e] : -INFINITY;
         if (!(ze == ze)) ze = -INFINITY;
-        vals[j] = ze;
+        raw[j] = scoring == 2 ? 1.0f / (1.0f + expf(-ze)) : ze;
+        vals[j] = e < E ? raw[j] + (correction ? correction[e] : 0.f) : -INFINITY;
     }
-    float best = 0.f, total = 0.f;
-    unsigned taken_mask = 0;        // bit j: this lane's expert lane + 64 j has been chosen
     if (mix_all) {                  // zeros first; the fence lets them land before lane 0 writes the chosen ones at the end
         for (int e = lane; e < E; e += WAVE) mix_all[static_cast<size_t>(t) * E + e] = 0.f;
         __threadfence_block();
@@ -512,86 +572,101 @@ __global__ void route_top_kernel(const float* __restrict__ z, int32_t* __restric
     unsigned long long open_groups = ~0ull;       // bit g: experts of group g may be chosen
     const int per_group = E / max(n_groups, 1);
     if (n_groups > 1) {
-        // lane g ends up with the largest logit of group g
+        // lane g ends up with the score of group g: the sum of its `group_top` largest scores
         float mine = -INFINITY;
         for (int g = 0; g < n_groups; ++g) {
-            float v = -INFINITY;
+            float sum = 0.f;
+            unsigned used = 0;      // bit j: this lane's expert lane + 64 j has been counted for this group
+            for (int n = 0; n < group_top; ++n) {
+                float v = -INFINITY;
+                int at = NO_EXPERT;
 #pragma unroll
-            for (int j = 0; j < SLOTS; ++j) {
-                const int e = lane + j * WAVE;
-                if (e < E && e / per_group == g) v = fmaxf(v, vals[j]);
+                for (int j = 0; j < SLOTS; ++j) {
+                    const int e = lane + j * WAVE;
+                    if (e < E && e / per_group == g && !((used >> j) & 1u) && (at == NO_EXPERT || vals[j] > v)) { at = e; v = vals[j]; }
+                }
+                const float vmax = wave_max(v);
+                const int cand = lowest_of((at != NO_EXPERT && v == vmax) ? at : NO_EXPERT);
+                if (cand == NO_EXPERT) break;             // a group of fewer experts than group_top (the same for all lanes)
+                if (cand % WAVE == lane) used |= 1u << (cand / WAVE);
+                sum += vmax;
             }
-            v = wave_max(v);
-            if (lane == g) mine = v;
+            if (lane == g) mine = sum;
         }
         open_groups = 0ull;
         bool used = lane >= n_groups;
         for (int k = 0; k < keep; ++k) {
             const float v = used ? -INFINITY : mine;
             const float vmax = wave_max(v);
-            int cand = (!used && v == vmax) ? lane : 0x7fffffff;
-#pragma unroll
-            for (int off = WAVE / 2; off > 0; off >>= 1) cand = min(cand, __shfl_xor(cand, off, WAVE));
-            if (cand == 0x7fffffff) break;        // unreachable: keep <= n_groups
+            const int cand = lowest_of((!used && v == vmax) ? lane : NO_EXPERT);
+            if (cand == NO_EXPERT) break;         // unreachable: keep <= n_groups
             if (cand == lane) used = true;
             open_groups |= 1ull << cand;
         }
     }
-    if (over_all) {                 // the softmax runs over every expert, chosen or not
+    float best = 0.f, total = 1.f;
+    if (scoring == 1) {             // the softmax runs over every expert, chosen or not
         float v = -INFINITY;
 #pragma unroll
-        for (int j = 0; j < SLOTS; ++j) v = fmaxf(v, vals[j]);
+        for (int j = 0; j < SLOTS; ++j) v = fmaxf(v, raw[j]);
         best = wave_max(v);
         float sum = 0.f;
 #pragma unroll
         for (int j = 0; j < SLOTS; ++j)
-            if (lane + j * WAVE < E && vals[j] > -INFINITY) sum += expf(vals[j] - best);
+            if (lane + j * WAVE < E && raw[j] > -INFINITY) sum += expf(raw[j] - best);
         total = wave_sum(sum);
     }
+    unsigned taken_mask = 0;        // bit j: this lane's expert lane + 64 j has been chosen
     for (int k = 0; k < top; ++k) {
         float v = -INFINITY;
-        int at = 0x7fffffff;
+        int at = NO_EXPERT;
 #pragma unroll
         for (int j = 0; j < SLOTS; ++j) {
             const int e = lane + j * WAVE;
             if (e >= E) continue;
             const bool taken = (taken_mask >> j) & 1u;
             const bool open = (open_groups >> (n_groups > 1 ? e / per_group : 0)) & 1ull;
-            if (!taken && open && (at == 0x7fffffff || vals[j] > v)) { at = e; v = vals[j]; }
+            if (!taken && open && (at == NO_EXPERT || vals[j] > v)) { at = e; v = vals[j]; }
         }
         const float vmax = wave_max(v);
-        int cand = (at != 0x7fffffff && v == vmax) ? at : 0x7fffffff;
-#pragma unroll
-        for (int off = WAVE / 2; off > 0; off >>= 1) cand = min(cand, __shfl_xor(cand, off, WAVE));
-        if (k == 0 && !over_all) best = vmax;
-        const float w = expf(vmax - best);
-        if (!over_all) total += w;
+        const int cand = lowest_of((at != NO_EXPERT && v == vmax) ? at : NO_EXPERT);
         if (cand % WAVE == lane) taken_mask |= 1u << (cand / WAVE);
-        if (lane == 0) { c[k] = cand; m[k] = w; }
+        float mine = 0.f;           // what weighs the chosen expert: only its owner has it
+#pragma unroll
+        for (int j = 0; j < SLOTS; ++j)
+            if (lane + j * WAVE == cand) mine = raw[j];
+        const float value = wave_sum(mine);
+        if (lane == 0) { c[k] = cand; m[k] = value; }
     }
     if (lane == 0) {
+        if (scoring == 0) {         // the softmax among the chosen
+            best = -INFINITY;
+            for (int k = 0; k < top; ++k) best = fmaxf(best, m[k]);
+            total = 0.f;
+            for (int k = 0; k < top; ++k) total += expf(m[k] - best);
+        }
         for (int k = 0; k < top; ++k) {
-            const float w = m[k] / total;
+            const float w = (scoring == 2 ? m[k] : expf(m[k] - best) / total) * route_scale;
             m[k] = w;
             if (mix_all) mix_all[static_cast<size_t>(t) * E + c[k]] = w;
         }
     }
 }
 
-NI_EXPORT int ni_route_top(const void* z, void* chosen, void* mix, void* mix_all, int T, int E, int top, int over_all,
-                           int n_groups, int keep, hipStream_t stream) {
+NI_EXPORT int ni_route_top(const void* z, const void* correction, void* chosen, void* mix, void* mix_all, int T, int E, int top,
+                           int scoring, int n_groups, int keep, int group_top, float route_scale, hipStream_t stream) {
     if (T <= 0) return 0;
-    if (top < 1 || top > E || E > 32 * WAVE) return -1;
+    if (top < 1 || top > E || E > 32 * WAVE || scoring < 0 || scoring > 2 || group_top < 1) return -1;
     if (n_groups < 1 || n_groups > WAVE || E % n_groups || keep < 1 || keep > n_groups || top > E / n_groups * keep) return -1;
     if (E <= WAVE)
-        route_top_kernel<1><<<T, WAVE, 0, stream>>>((const float*)z, (int32_t*)chosen, (float*)mix, (float*)mix_all, T, E, top,
-                                                    over_all, n_groups, keep);
+        route_top_kernel<1><<<T, WAVE, 0, stream>>>((const float*)z, (const float*)correction, (int32_t*)chosen, (float*)mix,
+                                                    (float*)mix_all, T, E, top, scoring, n_groups, keep, group_top, route_scale);
     else if (E <= 4 * WAVE)
-        route_top_kernel<4><<<T, WAVE, 0, stream>>>((const float*)z, (int32_t*)chosen, (float*)mix, (float*)mix_all, T, E, top,
-                                                    over_all, n_groups, keep);
+        route_top_kernel<4><<<T, WAVE, 0, stream>>>((const float*)z, (const float*)correction, (int32_t*)chosen, (float*)mix,
+                                                    (float*)mix_all, T, E, top, scoring, n_groups, keep, group_top, route_scale);
     else
-        route_top_kernel<32><<<T, WAVE, 0, stream>>>((const float*)z, (int32_t*)chosen, (float*)mix, (float*)mix_all, T, E, top,
-                                                     over_all, n_groups, keep);
+        route_top_kernel<32><<<T, WAVE, 0, stream>>>((const float*)z, (const float*)correction, (int32_t*)chosen, (float*)mix,
+                                                     (float*)mix_all, T, E, top, scoring, n_groups, keep, group_top, route_scale);
     return NI_LAUNCH_RESULT();
 }
 
@@ -642,21 +717,37 @@ __global__ void experts_act_vec_kernel(const T* __restrict__ up, const float* __
     VecIO<T, 8>::store(act + i, v);
 }
 
-// the gated form: an expert's rows of `up` are [gate: ff | up: ff], act[t, e * ff + i] = mix_all[t, e] * silu(gate) * up
+// What a gated hidden unit gives from its gate g and its up value u.  `form` 1: silu(g) * u.  `form` 2, the capped form:
+// g <- min(g, limit), u <- clamp(u, -limit, limit), then g * sigmoid(slope * g) * (u + 1).
+struct GluForm {
+    int form;
+    float limit, slope;
+};
+
+__device__ __forceinline__ float glu_value(float g, float u, const GluForm f) {
+    if (f.form == 2) {
+        g = fminf(g, f.limit);
+        u = fminf(fmaxf(u, -f.limit), f.limit);
+        return g / (1.0f + expf(-f.slope * g)) * (u + 1.0f);
+    }
+    return g / (1.0f + expf(-g)) * u;
+}
+
+// the gated forms: an expert's rows of `up` are [gate: ff | up: ff], act[t, e * ff + i] = mix_all[t, e] * glu(gate, up);
+// a null mix_all: every expert counts once (one feed-forward that every token uses is E = 1 of these)
 template <typename T>
 __global__ void experts_act_gated_kernel(const T* __restrict__ up, const float* __restrict__ mix_all, T* __restrict__ act,
-                                         int E, int ff, size_t n) {
+                                         int E, int ff, size_t n, GluForm form) {
     const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (i >= n) return;
     const size_t width = static_cast<size_t>(E) * ff;
     const size_t t = i / width;
     const int e = static_cast<int>((i % width) / ff), c = static_cast<int>(i % ff);
-    const float w = mix_all[t * E + e];
+    const float w = mix_all ? mix_all[t * E + e] : 1.f;
     float v = 0.f;
     if (w != 0.f) {
         const T* src = up + (t * E + e) * 2 * static_cast<size_t>(ff);
-        const float g = ld(src + c), u = ld(src + ff + c);
-        v = w * (g / (1.0f + expf(-g))) * u;
+        v = w * glu_value(ld(src + c), ld(src + ff + c), form);
     }
     st(act + i, v);
 }
@@ -665,7 +756,7 @@ __global__ void experts_act_gated_kernel(const T* __restrict__ up, const float* 
 // expert that was not chosen are not read at all
 template <typename T>
 __global__ void experts_act_gated_vec_kernel(const T* __restrict__ up, const float* __restrict__ mix_all, T* __restrict__ act,
-                                             int E, int ff, size_t pieces) {
+                                             int E, int ff, size_t pieces, GluForm form) {
     const size_t idx = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (idx >= pieces) return;
     const size_t i = idx * 8;
@@ -673,7 +764,7 @@ __global__ void experts_act_gated_vec_kernel(const T* __restrict__ up, const flo
     const size_t t = i / width;
     const size_t in_row = i - t * width;
     const int e = static_cast<int>(in_row / ff), c = static_cast<int>(in_row - static_cast<size_t>(e) * ff);
-    const float w = mix_all[t * E + e];
+    const float w = mix_all ? mix_all[t * E + e] : 1.f;
     float v[8];
     if (w != 0.f) {
         const T* src = up + (t * E + e) * 2 * static_cast<size_t>(ff) + c;
@@ -681,7 +772,7 @@ __global__ void experts_act_gated_vec_kernel(const T* __restrict__ up, const flo
         VecIO<T, 8>::load(src, g);
         VecIO<T, 8>::load(src + ff, u);
 #pragma unroll
-        for (int j = 0; j < 8; ++j) v[j] = w * (g[j] / (1.0f + expf(-g[j]))) * u[j];
+        for (int j = 0; j < 8; ++j) v[j] = w * glu_value(g[j], u[j], form);
     } else {
 #pragma unroll
         for (int j = 0; j < 8; ++j) v[j] = 0.f;
@@ -689,22 +780,26 @@ __global__ void experts_act_gated_vec_kernel(const T* __restrict__ up, const flo
     VecIO<T, 8>::store(act + i, v);
 }
 
-NI_EXPORT int ni_experts_act(const void* up, const void* mix_all, void* act, int T, int E, int ff, int gated, int dtype, hipStream_t stream) {
+// `gated` 0: relu(up)^2; 1: silu(gate) * up; 2: the capped form with `limit` and `slope` (see glu_value)
+NI_EXPORT int ni_experts_act(const void* up, const void* mix_all, void* act, int T, int E, int ff, int gated, float limit, float slope,
+                             int dtype, hipStream_t stream) {
     const size_t n = static_cast<size_t>(T) * E * ff;
     if (n == 0) return 0;
+    if (gated < 0 || gated > 2 || (!gated && !mix_all)) return -1;
+    const GluForm form{gated, limit, slope};
     if (gated && ff % 8 == 0 && aligned16(up, act)) {
         const size_t pieces = n / 8;
         if (dtype == 0)
-            experts_act_gated_vec_kernel<float><<<blocks_of(pieces, 256), 256, 0, stream>>>((const float*)up, (const float*)mix_all, (float*)act, E, ff, pieces);
+            experts_act_gated_vec_kernel<float><<<blocks_of(pieces, 256), 256, 0, stream>>>((const float*)up, (const float*)mix_all, (float*)act, E, ff, pieces, form);
         else
-            experts_act_gated_vec_kernel<bf16_t><<<blocks_of(pieces, 256), 256, 0, stream>>>((const bf16_t*)up, (const float*)mix_all, (bf16_t*)act, E, ff, pieces);
+            experts_act_gated_vec_kernel<bf16_t><<<blocks_of(pieces, 256), 256, 0, stream>>>((const bf16_t*)up, (const float*)mix_all, (bf16_t*)act, E, ff, pieces, form);
         return NI_LAUNCH_RESULT();
     }
     if (gated) {
         if (dtype == 0)
-            experts_act_gated_kernel<float><<<blocks_of(n, 256), 256, 0, stream>>>((const float*)up, (const float*)mix_all, (float*)act, E, ff, n);
+            experts_act_gated_kernel<float><<<blocks_of(n, 256), 256, 0, stream>>>((const float*)up, (const float*)mix_all, (float*)act, E, ff, n, form);
         else
-            experts_act_gated_kernel<bf16_t><<<blocks_of(n, 256), 256, 0, stream>>>((const bf16_t*)up, (const float*)mix_all, (bf16_t*)act, E, ff, n);
+            experts_act_gated_kernel<bf16_t><<<blocks_of(n, 256), 256, 0, stream>>>((const bf16_t*)up, (const float*)mix_all, (bf16_t*)act, E, ff, n, form);
         return NI_LAUNCH_RESULT();
     }
     if (ff % 8 == 0 && aligned16(up, act)) {
@@ -731,8 +826,8 @@ NI_EXPORT int ni_experts_act(const void* up, const void* mix_all, void* act, int
 // flight together, and the input row is read once for all of them.
 template <typename T, int R, bool GATED>
 __global__ void experts_up_few_kernel(const T* __restrict__ x, const T* __restrict__ w_up, const int32_t* __restrict__ chosen,
-                                      float* __restrict__ hid, int d, int ff, int top, bool vec) {
-    // GATED: an expert owns 2 ff rows of w_up, its gate rows and then its up rows; hid = silu(gate . x) * (up . x)
+                                      float* __restrict__ hid, int d, int ff, int top, bool vec, GluForm form) {
+    // GATED: an expert owns 2 ff rows of w_up, its gate rows and then its up rows; hid = glu(gate . x, up . x)
     const int pair = blockIdx.x;                 // t * top + k
     const int t = pair / top;
     const int e = chosen[pair];
@@ -776,7 +871,7 @@ __global__ void experts_up_few_kernel(const T* __restrict__ x, const T* __restri
         if (lane == 0 && i0 + u < ff) {
             float a;
             if constexpr (GATED) {
-                a = s[u] / (1.0f + expf(-s[u])) * s[R + u];
+                a = glu_value(s[u], s[R + u], form);
             } else {
                 a = fmaxf(s[u], 0.f);
                 a = a * a;
@@ -838,30 +933,33 @@ __global__ void experts_down_few_kernel(const float* __restrict__ hid, const T* 
 
 template <typename T, int R>
 static void launch_experts_few(const void* x, const void* w_up, const void* w_down, const void* chosen, const void* mix,
-                               void* hid, void* out, int T_, int d, int ff, int E, int top, bool gated, bool vec_up, bool vec_down,
+                               void* hid, void* out, int T_, int d, int ff, int E, int top, GluForm form, bool vec_up, bool vec_down,
                                hipStream_t stream) {
+    const bool gated = form.form != 0;
     constexpr int rows = 4 * R;                  // four wavefronts a workgroup
     dim3 g1(T_ * top, (ff + rows - 1) / rows), g2(T_, (d + rows - 1) / rows);
     if (gated)
-        experts_up_few_kernel<T, R, true><<<g1, 256, 0, stream>>>((const T*)x, (const T*)w_up, (const int32_t*)chosen, (float*)hid, d, ff, top, vec_up);
+        experts_up_few_kernel<T, R, true><<<g1, 256, 0, stream>>>((const T*)x, (const T*)w_up, (const int32_t*)chosen, (float*)hid, d, ff, top, vec_up, form);
     else
-        experts_up_few_kernel<T, R, false><<<g1, 256, 0, stream>>>((const T*)x, (const T*)w_up, (const int32_t*)chosen, (float*)hid, d, ff, top, vec_up);
+        experts_up_few_kernel<T, R, false><<<g1, 256, 0, stream>>>((const T*)x, (const T*)w_up, (const int32_t*)chosen, (float*)hid, d, ff, top, vec_up, form);
     experts_down_few_kernel<T, R><<<g2, 256, 0, stream>>>((const float*)hid, (const T*)w_down, (const int32_t*)chosen,
                                                           (const float*)mix, (float*)out, d, ff, E, top, vec_down);
 }
 
-// `gated` 0: w_up [E * ff, d], hid = relu(.)^2; 1: w_up [E * 2 ff, d] (an expert's gate rows, then its up rows),
-// hid = silu(gate) * up
+// `gated` 0: w_up [E * ff, d], hid = relu(.)^2; 1 or 2: w_up [E * 2 ff, d] (an expert's gate rows, then its up rows),
+// hid = silu(gate) * up, or the capped form with `limit` and `slope` (see glu_value)
 NI_EXPORT int ni_experts_few(const void* x, const void* w_up, const void* w_down, const void* chosen, const void* mix,
-                             void* hid, void* out, int T, int d, int ff, int E, int top, int gated, int dtype, hipStream_t stream) {
+                             void* hid, void* out, int T, int d, int ff, int E, int top, int gated, float limit, float slope,
+                             int dtype, hipStream_t stream) {
     if (T <= 0) return 0;
+    if (gated < 0 || gated > 2) return -1;
     // rows of whole 16-byte (bfloat16) or 32-byte (float32) pieces that start on such a piece are read in pieces
     const bool vec_up = d % 8 == 0 && aligned16(x, w_up);
     const bool vec_down = ff % 8 == 0 && aligned16(w_down, hid);
     // four rows a wavefront where that still leaves the second kernel a workgroup for every compute unit, else two
     // (the gated form walks twice the rows in its first kernel and keeps to two)
     const bool four = !gated && static_cast<long long>(T) * ((d + 15) / 16) >= 256;
-    const bool g = gated != 0;
+    const GluForm g{gated, limit, slope};
     if (dtype == 0) {
         if (four) launch_experts_few<float, 4>(x, w_up, w_down, chosen, mix, hid, out, T, d, ff, E, top, g, vec_up, vec_down, stream);
         else launch_experts_few<float, 2>(x, w_up, w_down, chosen, mix, hid, out, T, d, ff, E, top, g, vec_up, vec_down, stream);

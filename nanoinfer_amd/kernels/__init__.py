@@ -1187,7 +1187,8 @@ torch.backends.cudnn.allow_tf32 = False
 from .stream import (BIAS_ATTENTION_MFMA_FROM, DELTA_RUN_FROM, EXPERTS_FEW_ROWS, add_rmsnormed, add_vector,  # noqa: E402,F401
                      bias_attention, bias_attention_lib, bias_attention_mfma, bias_attention_mfma_rows, bias_attention_rows, bias_attention_runs, delta_rule, delta_rule_lib, embed_scaled, experts_act, experts_few,
                      gated_side, kv_store, route_top, stream_add, stream_lib, embed_pair_hash, add_rows_vector, qk_norm_rope_store,
-                     depth_mix, gate_heads, heads_apart, poly_norm, rmsnorm_cols, scale_, gate_rows, gather_pages, rows_to_pages)
+                     depth_mix, gate_heads, heads_apart, poly_norm, rmsnorm_cols, scale_, gate_rows, gather_pages, rows_to_pages,
+                     post_norm, EXPERT_FORMS, ROUTE_SCORINGS)
 # mixers with a state of fixed size: linear attention with a decay a head, the selective scan
 from .state import (conv_silu, decay_attention, decay_in_runs, decay_state_floats, gated_rmsnorm, scan_state_floats, selective_scan,  # noqa: E402,F401
                     silu_rows, state_mixers_lib, gated_memory, memory_norm, memory_state_floats)

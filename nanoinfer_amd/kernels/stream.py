@@ -142,6 +142,26 @@ def add_rmsnormed(h: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, eps: f
     return h
 
 
+def post_norm(h: torch.Tensor, addends: Optional[torch.Tensor], alpha: float, weight: torch.Tensor, eps: float,
+              x: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``h <- rmsnorm(alpha * h + sum of addends) * weight`` in place, all float32: the stream of a block whose norm stands
+    behind the sum.  ``addends`` float32 [T, d] or [S, T, d] (summed in their order), or None; ``x`` [T, d] in a compute
+    type takes a copy of the result for the products that read it next."""
+    T, d = h.shape
+    _gpu(h, "h", torch.float32)
+    _gpu(weight, "weight", torch.float32, (d,))
+    n = 0
+    if addends is not None:
+        _gpu(addends, "addends", torch.float32)
+        _need(addends.shape[-2:] == (T, d) and addends.dim() in (2, 3), "addends are float32 [T, d] or [S, T, d]")
+        n = 1 if addends.dim() == 2 else addends.shape[0]
+    if x is not None:
+        _gpu(x, "x", None, (T, d))
+    _check(stream_lib().ni_post_norm(_ptr(h), _ptr(addends), n, _float(alpha), _ptr(weight), _float(eps), _ptr(x),
+                                     0 if x is None else dtype_code(x.dtype), T, d, _stream()), "post_norm")
+    return h
+
+
 def rmsnorm_cols(rows: torch.Tensor, col: int, weight: torch.Tensor, eps: float, out_dtype: torch.dtype) -> torch.Tensor:
     """``x / sqrt(mean(x^2) + eps) * weight`` over the columns ``col .. col + len(weight)`` of ``rows`` float32 [T, wide]
     (some of a stacked product's accumulators); [T, len(weight)] in ``out_dtype``."""
@@ -185,29 +205,33 @@ def scale_(x: torch.Tensor, factor: float) -> torch.Tensor:
     return x
 
 
-def gate_heads(o: torch.Tensor, gate_rows: torch.Tensor, gate_col: int, out_dtype: torch.dtype) -> torch.Tensor:
+def gate_heads(o: torch.Tensor, gate_rows: torch.Tensor, gate_col: int, out_dtype: torch.dtype, per_head: bool = False) -> torch.Tensor:
     """``y[t, h * dv + c] = o[h, t, c] * sigmoid(gate[t, h * dv + c])``: ``o`` float32 [H, T, dv] (head by head), the
-    gate's pre-activations the columns ``gate_col ..`` of ``gate_rows`` float32 [T, wide]; y [T, H * dv] in ``out_dtype``."""
+    gate's pre-activations the columns ``gate_col ..`` of ``gate_rows`` float32 [T, wide]; y [T, H * dv] in ``out_dtype``.
+    ``per_head``: one gate a head, ``gate[t, h]``."""
     H, T, dv = o.shape
+    per = dv if per_head else 1
     _gpu(o, "o", torch.float32)
     _gpu(gate_rows, "gate_rows", torch.float32)
-    _need(gate_rows.shape[0] == T and 0 <= gate_col and gate_col + H * dv <= gate_rows.shape[1], "the gate's columns lie outside its rows")
+    _need(gate_rows.shape[0] == T and 0 <= gate_col and gate_col + H * dv // per <= gate_rows.shape[1], "the gate's columns lie outside its rows")
     y = torch.empty(T, H * dv, dtype=out_dtype, device=o.device)
     gate = ctypes.c_void_p(gate_rows.data_ptr() + 4 * gate_col)
-    _check(stream_lib().ni_gate_heads(_ptr(o), gate, gate_rows.shape[1], _ptr(y), T, H, dv, dtype_code(out_dtype), _stream()), "gate_heads")
+    _check(stream_lib().ni_gate_heads(_ptr(o), gate, gate_rows.shape[1], _ptr(y), T, H, dv, per, dtype_code(out_dtype), _stream()), "gate_heads")
     return y
 
 
-def gate_rows(x: torch.Tensor, gate_rows_: torch.Tensor, gate_col: int, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """``y[t, j] = x[t, j] * sigmoid(gate[t, j])``: ``x`` [T, n] in the compute type, the gate's pre-activations the
-    columns ``gate_col ..`` of ``gate_rows_`` float32 [T, wide]; y like x."""
+def gate_rows(x: torch.Tensor, gate_rows_: torch.Tensor, gate_col: int, out: Optional[torch.Tensor] = None, every: int = 1) -> torch.Tensor:
+    """``y[t, j] = x[t, j] * sigmoid(gate[t, j // every])``: ``x`` [T, n] in the compute type, the gate's pre-activations
+    the columns ``gate_col ..`` of ``gate_rows_`` float32 [T, wide]; y like x.  ``every`` 1: a gate a channel; a head's
+    channels: a gate a head."""
     T, n = x.shape
     _gpu(x, "x")
     _gpu(gate_rows_, "gate_rows", torch.float32)
-    _need(gate_rows_.shape[0] == T and 0 <= gate_col and gate_col + n <= gate_rows_.shape[1], "the gate's columns lie outside its rows")
+    _need(every >= 1 and n % every == 0, "whole groups of channels share a gate")
+    _need(gate_rows_.shape[0] == T and 0 <= gate_col and gate_col + n // every <= gate_rows_.shape[1], "the gate's columns lie outside its rows")
     y = torch.empty_like(x) if out is None else out
     gate = ctypes.c_void_p(gate_rows_.data_ptr() + 4 * gate_col)
-    _check(stream_lib().ni_gate_rows(_ptr(x), gate, gate_rows_.shape[1], _ptr(y), T, n, dtype_code(x.dtype), _stream()), "gate_rows")
+    _check(stream_lib().ni_gate_rows(_ptr(x), gate, gate_rows_.shape[1], _ptr(y), T, n, int(every), dtype_code(x.dtype), _stream()), "gate_rows")
     return y
 
 
@@ -251,36 +275,67 @@ def heads_apart(x: torch.Tensor, H: int, n: int) -> torch.Tensor:
 
 # ------------------------------------------------------------------ router and experts
 
-def route_top(z: torch.Tensor, top: int, mix_all: bool, over_all: bool = False, groups: int = 1, keep: int = 1):
-    """The ``top`` largest logits of every row of ``z`` float32 [T, E] and their weights: the softmax among the
-    chosen, or (``over_all``) the softmax over all E experts, not renormalised.  With ``groups`` > 1 the experts
-    form that many equal groups of neighbours, a group counts as much as its largest logit, and only experts of the
-    ``keep`` best groups can be chosen.
-    ``(chosen int32 [T, top], mix float32 [T, top], mix over all experts float32 [T, E] or None)``."""
+ROUTE_SCORINGS = {"softmax_chosen": 0, "softmax_all": 1, "sigmoid": 2}
+
+
+def route_top(z: torch.Tensor, top: int, mix_all: bool, over_all: bool = False, groups: int = 1, keep: int = 1,
+              scoring: Optional[str] = None, correction: Optional[torch.Tensor] = None, group_top: int = 1, scale: float = 1.0):
+    """The ``top`` experts of every row of ``z`` float32 [T, E] and their weights.  ``scoring``: "softmax_chosen" (an
+    expert's value is its logit, the weights the softmax among the chosen; the default), "softmax_all" (``over_all``:
+    the softmax over all E experts, not renormalised) or "sigmoid" (the value is ``sigmoid(logit)``, the weights the
+    values themselves); every weight times ``scale``.  ``correction`` float32 [E] is added to the values that choose,
+    never to the weights.  With ``groups`` > 1 the experts form that many equal groups of neighbours, a group counts as
+    much as the sum of its ``group_top`` largest choosing values, and only experts of the ``keep`` best groups can be
+    chosen.  ``(chosen int32 [T, top], mix float32 [T, top], mix over all experts float32 [T, E] or None)``."""
     T, E = z.shape
     _gpu(z, "z", torch.float32)
+    if scoring is None:
+        scoring = "softmax_all" if over_all else "softmax_chosen"
+    _need(scoring in ROUTE_SCORINGS, f"scoring {scoring!r} is not one of {sorted(ROUTE_SCORINGS)}")
     _need(1 <= top <= E, f"{top} of {E} experts cannot be chosen")
     _need(1 <= groups <= 64 and E % groups == 0 and 1 <= keep <= groups and top <= E // groups * keep,
           f"{top} experts cannot be chosen from {keep} of {groups} groups of {E} experts")
+    _need(group_top >= 1, "a group counts by at least one of its experts")
+    if correction is not None:
+        _gpu(correction, "correction", torch.float32, (E,))
     chosen = torch.empty(T, top, dtype=torch.int32, device=z.device)
     mix = torch.empty(T, top, dtype=torch.float32, device=z.device)
     dense = torch.empty(T, E, dtype=torch.float32, device=z.device) if mix_all else None
-    _check(stream_lib().ni_route_top(_ptr(z), _ptr(chosen), _ptr(mix), _ptr(dense), T, E, top, int(bool(over_all)),
-                                     int(groups), int(keep), _stream()), "route_top")
+    _check(stream_lib().ni_route_top(_ptr(z), _ptr(correction), _ptr(chosen), _ptr(mix), _ptr(dense), T, E, top,
+                                     ROUTE_SCORINGS[scoring], int(groups), int(keep), int(group_top), _float(scale), _stream()), "route_top")
     return chosen, mix, dense
 
 
-def experts_act(up: torch.Tensor, mix_all: torch.Tensor, ff: int, gated: bool = False) -> torch.Tensor:
-    """``mix_all[t, e] * relu(up[t, e * ff + i])^2`` in the type of ``up``; ``gated``: an expert's columns of ``up``
-    are [gate: ff | up: ff] and the result is ``mix_all[t, e] * silu(gate) * up``, [T, E * ff]."""
+EXPERT_FORMS = {"relu2": 0, "swiglu": 1, "capped_glu": 2}
+
+
+def _expert_form(gated) -> int:
+    """The number the kernels know an expert's activation by; ``gated`` may be a bool (relu2 / swiglu) or a name."""
+    if isinstance(gated, str):
+        _need(gated in EXPERT_FORMS, f"expert activation {gated!r} is not one of {sorted(EXPERT_FORMS)}")
+        return EXPERT_FORMS[gated]
+    return int(bool(gated))
+
+
+def experts_act(up: torch.Tensor, mix_all: Optional[torch.Tensor], ff: int, gated=False, limit: float = 0.0,
+                slope: float = 1.0) -> torch.Tensor:
+    """``mix_all[t, e] * relu(up[t, e * ff + i])^2`` in the type of ``up``; ``gated`` (True or "swiglu"): an expert's
+    columns of ``up`` are [gate: ff | up: ff] and the result is ``mix_all[t, e] * silu(gate) * up``, [T, E * ff];
+    "capped_glu": ``g = min(gate, limit)``, ``u = clamp(up, -limit, limit)``, ``mix * g * sigmoid(slope * g) * (u + 1)``.
+    ``mix_all`` None (gated forms): every expert counts once."""
     T, width = up.shape
-    E = mix_all.shape[1]
+    form = _expert_form(gated)
     _gpu(up, "up")
-    _gpu(mix_all, "mix_all", torch.float32, (T, E))
-    _need(width == E * ff * (2 if gated else 1), "the experts' hidden rows do not match the router")
+    if mix_all is None:
+        _need(form != 0 and width % (2 * ff) == 0, "without a mix the rows are whole gated experts")
+        E = width // (2 * ff)
+    else:
+        E = mix_all.shape[1]
+        _gpu(mix_all, "mix_all", torch.float32, (T, E))
+    _need(width == E * ff * (2 if form else 1), "the experts' hidden rows do not match the router")
     act = torch.empty(T, E * ff, dtype=up.dtype, device=up.device)
-    _check(stream_lib().ni_experts_act(_ptr(up), _ptr(mix_all), _ptr(act), T, E, ff, int(bool(gated)), dtype_code(up.dtype), _stream()),
-           "experts_act")
+    _check(stream_lib().ni_experts_act(_ptr(up), _ptr(mix_all), _ptr(act), T, E, ff, form, _float(limit), _float(slope),
+                                       dtype_code(up.dtype), _stream()), "experts_act")
     return act
 
 
@@ -288,13 +343,14 @@ EXPERTS_FEW_ROWS = 16       # up to here only the chosen experts' matrices are r
 
 
 def experts_few(x: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor, chosen: torch.Tensor, mix: torch.Tensor,
-                ff: int, gated: bool = False, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                ff: int, gated=False, out: Optional[torch.Tensor] = None, limit: float = 0.0, slope: float = 1.0) -> torch.Tensor:
     """The weighted sum of the chosen experts for a few rows: ``w_up`` [E * ff, d] (``gated``: [E * 2 ff, d], an
-    expert's gate rows and then its up rows; the hidden row is then ``silu(gate) * up`` instead of ``relu(up)^2``),
-    ``w_down`` [d, E * ff]; returns float32 [T, d] (``out``, if given)."""
+    expert's gate rows and then its up rows; the hidden row is then ``silu(gate) * up`` instead of ``relu(up)^2``, or,
+    "capped_glu", the capped form of :func:`experts_act`), ``w_down`` [d, E * ff]; returns float32 [T, d] (``out``, if given)."""
     T, d = x.shape
     top = chosen.shape[1]
-    per = ff * (2 if gated else 1)
+    form = _expert_form(gated)
+    per = ff * (2 if form else 1)
     E = w_up.shape[0] // per
     _gpu(x, "x", w_up.dtype)
     _gpu(w_up, "w_up", None, (E * per, d))
@@ -307,7 +363,8 @@ def experts_few(x: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor, chose
     else:
         _gpu(out, "out", torch.float32, (T, d))
     _check(stream_lib().ni_experts_few(_ptr(x), _ptr(w_up), _ptr(w_down), _ptr(chosen), _ptr(mix), _ptr(hid), _ptr(out),
-                                       T, d, ff, E, top, int(bool(gated)), dtype_code(x.dtype), _stream()), "experts_few")
+                                       T, d, ff, E, top, form, _float(limit), _float(slope), dtype_code(x.dtype), _stream()),
+           "experts_few")
     return out
 
 
@@ -414,47 +471,65 @@ def kv_store(qkv: torch.Tensor, k_off: int, v_off: int, slot_mapping: torch.Tens
 
 def qk_norm_rope_store(proj: torch.Tensor, positions: torch.Tensor, slot_mapping: Optional[torch.Tensor],
                        q_norm: Optional[torch.Tensor], k_norm: Optional[torch.Tensor], eps: float, freq: Optional[torch.Tensor],
-                       amplitude: float, q_out: Optional[torch.Tensor], kpool: torch.Tensor, vpool: torch.Tensor, H: int,
-                       values_are_keys: bool = False, col: int = 0) -> Optional[torch.Tensor]:
-    """From ``proj`` float32 [T, H*dk + G*dk + G*dv] (q | k | v as projected): the RMS norm over a token's WHOLE
-    query projection and over its whole key projection (weights ``q_norm`` [H*dk], ``k_norm`` [G*dk]; None: no norm),
+                       amplitude: float, q_out: Optional[torch.Tensor], kpool: Optional[torch.Tensor], vpool: Optional[torch.Tensor],
+                       H: int, values_are_keys: bool = False, col: int = 0, per_head: bool = False, adjacent: bool = False,
+                       q_dim: Optional[int] = None, rot_at_q: int = 0, rot_at_k: int = 0, k_normed: Optional[int] = None,
+                       queries_only: bool = False) -> Optional[torch.Tensor]:
+    """From ``proj`` float32 [T, H*dq + G*dk + G*dv] (q | k | v as projected): the RMS norm over a token's WHOLE
+    query projection and over its whole key projection (weights ``q_norm`` [H*dq], ``k_norm`` [G*dk]; None: no norm),
     then the rotation of the first ``2 * len(freq)`` channels of every head, channel c with channel c + len(freq), by
     ``position * freq[c]`` with cos and sin times ``amplitude`` (``freq`` None: no rotation), all in float32.  Queries
-    go to ``q_out`` [T, H*dk], keys and values into their page slots (``slot_mapping`` None: nothing is stored).
+    go to ``q_out`` [T, H*dq], keys and values into their page slots (``slot_mapping`` None: nothing is stored).
     ``values_are_keys``: ``proj`` is q | k alone and the keys as projected, before their norm, are stored as the values.
     ``H`` may be 0 (``q_out`` None): keys alone, and values may have no channels.  ``col``: the projections are the
-    columns from ``col`` on of wider rows."""
+    columns from ``col`` on of wider rows.
+
+    ``per_head``: every head is normed on its own, with one weight shared by the heads (``q_norm`` [dq], ``k_norm``
+    [k_normed]); of a key head only the first ``k_normed`` channels are normed then (default: all), the others pass as
+    projected.  ``adjacent``: the rotation pairs channel 2p with channel 2p + 1.  ``rot_at_q``, ``rot_at_k``: the first
+    rotated channel of a query head and of a key head.  ``q_dim``: a query head's size where it differs from a key
+    head's.  ``queries_only``: ``proj`` holds the queries alone (the pools only say the sizes, or are None)."""
     T, wide = proj.shape
-    width = (H + kpool.shape[1]) * kpool.shape[3] + (0 if values_are_keys else kpool.shape[1] * vpool.shape[3])
+    if queries_only:
+        G, dk, dv, ps = 0, 0, 0, 1
+        _need(slot_mapping is None, "queries alone leave nothing to store")
+    else:
+        pages, G, ps, dk = kpool.shape
+        dv = vpool.shape[3]
+    dq = dk if q_dim is None else int(q_dim)
+    _need(not queries_only or q_dim is not None, "queries alone need their head size")
+    width = H * dq + G * dk + (0 if values_are_keys else G * dv)
     _need(0 <= col and col + width <= wide, "the projections lie outside the rows")
-    if col == 0:
-        width = wide
-    pages, G, ps, dk = kpool.shape
-    dv = vpool.shape[3]
     _gpu(proj, "proj", torch.float32)
-    _need(width == (H + G) * dk + (0 if values_are_keys else G * dv), "proj is not q | k | v of these sizes")
     _need(not values_are_keys or dv == dk, "values that are the keys have the keys' size")
     _gpu(positions, "positions", torch.int32, (T,))
     if slot_mapping is not None:
         _gpu(slot_mapping, "slot_mapping", torch.int32, (T,))
+    normed = dk if k_normed is None else int(k_normed)
+    _need(0 <= normed <= dk and (per_head or normed == dk), "only norms a head keep some of a key's channels out")
     if q_norm is not None:
-        _gpu(q_norm, "q_norm", torch.float32, (H * dk,))
+        _gpu(q_norm, "q_norm", torch.float32, (dq,) if per_head else (H * dq,))
     if k_norm is not None:
-        _gpu(k_norm, "k_norm", torch.float32, (G * dk,))
+        _gpu(k_norm, "k_norm", torch.float32, (normed,) if per_head else (G * dk,))
     rot = 0
     if freq is not None:
         rot = 2 * freq.shape[0]
         _gpu(freq, "freq", torch.float32, (rot // 2,))
-        _need(0 < rot <= dk, f"{rot} rotated channels do not fit a head of {dk}")
-    _gpu(kpool, "kpool")
-    _gpu(vpool, "vpool", kpool.dtype, (pages, G, ps, dv))
+        _need(rot > 0 and (H == 0 or rot_at_q + rot <= dq) and (G == 0 or rot_at_k + rot <= dk) and rot_at_q >= 0 and rot_at_k >= 0,
+              f"{rot} rotated channels do not fit the heads")
+    dtype = q_out.dtype if queries_only else kpool.dtype
+    if not queries_only:
+        _gpu(kpool, "kpool")
+        _gpu(vpool, "vpool", kpool.dtype, (pages, G, ps, dv))
     if H > 0 or q_out is not None:
-        _gpu(q_out, "q_out", kpool.dtype, (T, H * dk))
+        _gpu(q_out, "q_out", dtype, (T, H * dq))
     src = ctypes.c_void_p(proj.data_ptr() + 4 * col)
     _check(bias_attention_lib().ni_qk_norm_rope_store(src, wide, _ptr(positions), _ptr(slot_mapping), _ptr(q_norm),
                                                       _ptr(k_norm), _float(eps), _ptr(freq), rot, _float(amplitude), _ptr(q_out),
-                                                      _ptr(kpool), _ptr(vpool), T, H, G, dk, dv, ps, int(bool(values_are_keys)),
-                                                      dtype_code(kpool.dtype), _stream()), "qk_norm_rope_store")
+                                                      _ptr(None if queries_only else kpool), _ptr(None if queries_only else vpool),
+                                                      T, H, G, dq, dk, dv, ps, int(bool(values_are_keys)), int(bool(per_head)),
+                                                      normed, int(rot_at_q), int(rot_at_k), int(bool(adjacent)),
+                                                      dtype_code(dtype), _stream()), "qk_norm_rope_store")
     return q_out
 
 
@@ -462,7 +537,7 @@ def bias_attention(qkv: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor, 
                    tiles: torch.Tensor, positions: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor, H: int, scale: float,
                    temp_coef: float, temp_every: int, heads_per_chunk: int, n_runs: int = 1,
                    workspace: Optional[torch.Tensor] = None, waves: int = 4, window: Optional[int] = None, keep_first: int = 0,
-                   out_scale: float = 1.0) -> torch.Tensor:
+                   out_scale: float = 1.0, sink: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Causal attention of the query heads in the first ``H * dk`` columns of ``qkv`` over the paged cache.
     ``tiles`` int32 [n, 4]: (sequence, first row, tokens, -) with tokens * heads of a chunk <= 16, the tokens of a
     tile being consecutive ones of one sequence; ``positions`` int32 [T] the position of every row;
@@ -470,7 +545,8 @@ def bias_attention(qkv: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor, 
     cut into that many runs, which meet in ``workspace`` (float32, at least T * H * n_runs * (dv + 2)) and are merged
     by a second kernel.  ``waves`` (1 to 4): wavefronts of a workgroup, four rows each; fewer than four only where no
     tile has more rows than they take.  ``window`` n: a query sees its last n keys (its own among them) and the first
-    ``keep_first`` keys of its sequence; ``out_scale`` multiplies the output."""
+    ``keep_first`` keys of its sequence; ``out_scale`` multiplies the output.  ``sink`` float32 [H]: one more term
+    ``exp(sink[head])`` in every row's denominator, with no key and no value."""
     T, width = qkv.shape
     pages, G, ps, dk = kpool.shape
     dv = vpool.shape[3]
@@ -493,6 +569,8 @@ def bias_attention(qkv: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor, 
     _need(1 <= heads_per_chunk <= 16, "heads_per_chunk")
     _need(1 <= n_runs <= 64, "n_runs")
     _need(1 <= waves <= 4, "waves")
+    if sink is not None:
+        _gpu(sink, "sink", torch.float32, (H,))
     if n_runs > 1:
         _need(workspace is not None and workspace.is_cuda and workspace.dtype == torch.float32 and workspace.is_contiguous()
               and workspace.numel() >= T * H * n_runs * (dv + 2), "the runs need a float32 workspace of T * H * n_runs * (dv + 2)")
@@ -500,7 +578,7 @@ def bias_attention(qkv: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor, 
                                                  block_table.shape[1], _ptr(tiles), tiles.shape[0], _ptr(positions), _ptr(bias), distances,
                                                  _ptr(out), H, G, dk, dv, ps, _float(scale), _float(temp_coef), int(temp_every),
                                                  heads_per_chunk, n_runs, _ptr(workspace if n_runs > 1 else None), T, waves,
-                                                 int(window or 0), int(keep_first), _float(out_scale),
+                                                 int(window or 0), int(keep_first), _float(out_scale), _ptr(sink),
                                                  dtype_code(qkv.dtype), _stream())
     if err == -2:
         raise KernelError(f"keys of {dk} and values of {dv} channels do not fit the kernel's staging memory")
@@ -521,7 +599,7 @@ def bias_attention_mfma_rows(dk: int, dv: int, one_pool: bool = False) -> int:
 def bias_attention_mfma(qkv: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor, block_table: torch.Tensor,
                         tiles: torch.Tensor, positions: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor, H: int,
                         scale: float, temp_coef: float, temp_every: int, heads_per_chunk: int, window: Optional[int] = None,
-                        keep_first: int = 0, out_scale: float = 1.0) -> torch.Tensor:
+                        keep_first: int = 0, out_scale: float = 1.0, sink: Optional[torch.Tensor] = None) -> torch.Tensor:
     """:func:`bias_attention` for steps with portions of prompts: tiles of up to 64 rows (tokens * heads of a chunk),
     both products on the float32 matrix instructions, the same formula and the same 32-bit softmax; no runs."""
     T, width = qkv.shape
@@ -540,6 +618,8 @@ def bias_attention_mfma(qkv: torch.Tensor, kpool: torch.Tensor, vpool: torch.Ten
     _need(bias_attention_mfma_rows(dk, dv, kpool.data_ptr() == vpool.data_ptr()) > 0,
           f"keys of {dk} and values of {dv} channels are not taken by the matrix-core kernel")
     _need(1 <= heads_per_chunk <= 64, "heads_per_chunk")
+    if sink is not None:
+        _gpu(sink, "sink", torch.float32, (H,))
     distances = 0
     if bias is not None:
         distances = bias.shape[0]
@@ -549,6 +629,6 @@ def bias_attention_mfma(qkv: torch.Tensor, kpool: torch.Tensor, vpool: torch.Ten
                                                        block_table.shape[1], _ptr(tiles), tiles.shape[0], _ptr(positions),
                                                        _ptr(bias), distances, _ptr(out), H, G, dk, dv, ps, _float(scale),
                                                        _float(temp_coef), int(temp_every), heads_per_chunk,
-                                                       int(window or 0), int(keep_first), _float(out_scale),
+                                                       int(window or 0), int(keep_first), _float(out_scale), _ptr(sink),
                                                        dtype_code(qkv.dtype), _stream()), "bias_attention_mfma")
     return out

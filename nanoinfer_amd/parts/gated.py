@@ -95,96 +95,167 @@ class LatentAttention(Part):
     weights reads the latents that another entry of the order wrote (``LayerRun.writes_cache`` False), with its own
     W_uk, W_uv, queries and window.
 
+    With ``rot_dim`` r > 0 positions enter through r more channels: ``W_dkv`` has ``rank + r`` rows, of which the last r,
+    not normed, are rotated (``position``: a PartSpec of family ``position``; ``adjacent_pairs``: channel 2i turns with
+    channel 2i + 1) and kept in the pages behind the latent, one key part for all heads; a query head is ``key_dim``
+    channels that meet ``W_uk[h] c`` and r rotated ones that meet that part; the two dot products are summed before the
+    scale.  The kernel's key is then the whole row ``[c | k_rot]`` and a query as the row sees it ``[W_uk[h]^T q_h |
+    q_rot]``; the r extra value channels meet zero rows of W_uv.
+
     Steps whose longest portion has ``expand_from`` tokens or more (and that are not recorded) take the other way:
     ``k_h`` and ``v_h`` of every latent the step can see are written out once for the step, and attention runs over H
-    heads of ``key_dim`` and ``value_dim`` channels, a fraction of the products where the latent is wider than a head.
+    heads of ``key_dim + rot_dim`` and ``value_dim`` channels, a fraction of the products where the latent is wider than a head.
 
-    params: hidden_size, num_heads, key_dim, value_dim, q_rank, rank, scale, window (None: every earlier key), eps,
-    expand_from (default ``LATENT_EXPAND_FROM``; None: never; it is never taken where ``rank < key_dim + value_dim``).
-    weights: dq [q_rank, d], dq_norm [q_rank], uq [H*dk, q_rank], dkv [rank, d] and dkv_norm [rank] (both or neither),
-    uk [H*dk, rank], uv [H*dv, rank], g [H*dv, d], o [d, H*dv]."""
+    params: hidden_size, num_heads, key_dim, value_dim, q_rank (None: the queries are ``W_q x``, no latent of their own),
+    rank, scale, window (None: every earlier key), eps, rot_dim (default 0), position, adjacent_pairs, gate ("channel", the
+    default: a gate a value channel; "head": one a head), expand_from (default ``LATENT_EXPAND_FROM``; None: never; it is
+    never taken where ``rank + rot_dim < key_dim + rot_dim + value_dim``).
+    weights: dq [q_rank, d], dq_norm [q_rank], uq [H*(dk+r), q_rank] (or q [H*(dk+r), d]), dkv [rank + r, d] and dkv_norm
+    [rank] (both or neither), uk [H*dk, rank], uv [H*dv, rank], g [H*dv, d] (or [H, d]), o [d, H*dv], sink [H] (absent:
+    none; one more term ``exp(sink[h])`` in the softmax's denominator)."""
 
     graph_safe = True
 
     @classmethod
     def weight_requests(cls, spec):
         p, w = spec.params, spec.weights
-        d, H, dk, dv, rq, r = p["hidden_size"], p["num_heads"], p["key_dim"], p["value_dim"], p["q_rank"], p["rank"]
-        out = [WeightRequest(w["dq"], (rq, d)), WeightRequest(w["dq_norm"], (rq,)), WeightRequest(w["uq"], (H * dk, rq)),
-               WeightRequest(w["uk"], (H * dk, r)), WeightRequest(w["uv"], (H * dv, r)), WeightRequest(w["g"], (H * dv, d)),
+        d, H, dk, dv, rq, r = p["hidden_size"], p["num_heads"], p["key_dim"], p["value_dim"], p.get("q_rank"), p["rank"]
+        dr = int(p.get("rot_dim", 0))
+        gates = H if p.get("gate", "channel") == "head" else H * dv
+        out = [WeightRequest(w["uk"], (H * dk, r)), WeightRequest(w["uv"], (H * dv, r)), WeightRequest(w["g"], (gates, d)),
                WeightRequest(w["o"], (d, H * dv))]
+        if rq is None:
+            out.append(WeightRequest(w["q"], (H * (dk + dr), d)))
+        else:
+            out += [WeightRequest(w["dq"], (rq, d)), WeightRequest(w["dq_norm"], (rq,)), WeightRequest(w["uq"], (H * (dk + dr), rq))]
         if "dkv" in w:
-            out += [WeightRequest(w["dkv"], (r, d)), WeightRequest(w["dkv_norm"], (r,))]
+            out += [WeightRequest(w["dkv"], (r + dr, d)), WeightRequest(w["dkv_norm"], (r,))]
+        if "sink" in w:
+            out.append(WeightRequest(w["sink"], (H,)))
+        if p.get("position") is not None:
+            from .standard import requests_of
+            out += requests_of("position", p["position"])
         return out
 
     def __init__(self, spec, weights, rt):
         super().__init__(spec, weights, rt)
         p, names = spec.params, spec.weights
         self.H, self.dk, self.dv = int(p["num_heads"]), int(p["key_dim"]), int(p["value_dim"])
-        self.q_rank, self.rank = int(p["q_rank"]), int(p["rank"])
+        self.q_rank = None if p.get("q_rank") is None else int(p["q_rank"])
+        self.rank, self.dr = int(p["rank"]), int(p.get("rot_dim", 0))
+        self.row, self.dq = self.rank + self.dr, self.dk + self.dr       # what a token keeps; a query head
         self.window = None if p.get("window") is None else int(p["window"])
         self.eps = float(p["eps"])
         self.own = "dkv" in names
-        # one product for everything that reads the layer's input: the queries' latent, the gate, and the latent
-        # of keys and values if this layer makes its own; float32 out (norms and the gate read the accumulators)
-        first = ["dq", "g"] + (["dkv"] if self.own else [])
-        self.gate_col = self.q_rank
-        self.latent_col = self.q_rank + self.H * self.dv
+        gate = p.get("gate", "channel")
+        if gate not in ("channel", "head"):
+            raise ValueError(f"gate {gate!r} is not 'channel' or 'head'")
+        self.gate_per_head = gate == "head"
+        H, dk, dv, dr, rank, row = self.H, self.dk, self.dv, self.dr, self.rank, self.row
+        if row > 256:
+            raise ValueError(f"a latent of {rank} + {dr} channels is more than the attention kernels' 256 value channels")
+        self.freq, self.amplitude, self.adjacent = None, 1.0, bool(p.get("adjacent_pairs", False))
+        if dr:
+            from .standard import build_part
+            if p.get("position") is None:
+                raise ValueError("rotated channels need a position part")
+            self.freq, self.amplitude = build_part("position", p["position"], getattr(weights, "checkpoint", {}), rt).frequencies()
+            if 2 * self.freq.shape[0] != dr:
+                raise ValueError(f"{2 * self.freq.shape[0]} rotated channels, rot_dim is {dr}")
+        # one product for everything that reads the layer's input: the queries (or their latent), the latent of keys and
+        # values with its rotated part if this layer makes its own, and the gate; float32 out (norms, rotation and the
+        # gate read the accumulators)
+        first = ["q" if self.q_rank is None else "dq"] + (["dkv"] if self.own else []) + ["g"]
+        self.latent_col = int(weights[first[0]].shape[0])
+        self.gate_col = self.latent_col + (row if self.own else 0)
         self.w_in = rt.weight("|".join(names[k] for k in first), torch.cat([weights[k] for k in first], dim=0))
-        self.dq_norm = rt.vector32(names["dq_norm"], weights["dq_norm"])
         self.dkv_norm = rt.vector32(names["dkv_norm"], weights["dkv_norm"]) if self.own else None
-        self.w_uq = rt.weight(names["uq"], weights["uq"])
+        self.dq_norm = self.w_uq = None
+        if self.q_rank is not None:
+            self.dq_norm = rt.vector32(names["dq_norm"], weights["dq_norm"])
+            self.w_uq = rt.weight(names["uq"], weights["uq"])
         self.w_o = rt.weight(names["o"], weights["o"])
-        # per head: [dk, rank] for the queries' side, [rank, dv] behind the softmax
-        self.uk = rt.matrix(names["uk"], weights["uk"]).view(self.H, self.dk, self.rank)
-        self.uv_t = rt.matrix(names["uv"], weights["uv"]).view(self.H, self.dv, self.rank).transpose(1, 2)
-        self.core = PagedSoftmax(self.H, 1, self.rank, self.rank, float(p["scale"]), one_pool=True)
+        self.sink = rt.vector32(names["sink"], weights["sink"]) if "sink" in names else None
+        # per head: [dk + dr, rank + dr] for the queries' side (W_uk[h], and an identity that hands the rotated channels
+        # on), [rank + dr, dv] behind the softmax (W_uv[h]^T over zero rows)
+        uk = torch.zeros(H, self.dq, row, dtype=weights["uk"].dtype)
+        uk[:, :dk, :rank] = weights["uk"].view(H, dk, rank)
+        uv = torch.zeros(H, dv, row, dtype=weights["uv"].dtype)
+        uv[:, :, :rank] = weights["uv"].view(H, dv, rank)
+        if dr:
+            uk[:, dk:, rank:] = torch.eye(dr, dtype=uk.dtype)
+        self.uk = rt.matrix(names["uk"] + "|row", uk.view(H * self.dq, row)).view(H, self.dq, row)
+        self.uv_t = rt.matrix(names["uv"] + "|row", uv.view(H * dv, row)).view(H, dv, row).transpose(1, 2)
+        self.core = PagedSoftmax(H, 1, row, row, float(p["scale"]), one_pool=True, sink=self.sink)
         # steps with long portions: keys and values of every head are made of the latents the step can see, once,
         # and attention runs at the heads' own sizes
         self.expand_from = p.get("expand_from", LATENT_EXPAND_FROM)
-        if self.rank < self.dk + self.dv:      # attention over the latents is then the smaller sum of products already
+        if row < self.dq + dv:      # attention over the latents is then the smaller sum of products already
             self.expand_from = None
         if self.expand_from is not None:
             self.expand_from = max(2, int(self.expand_from))
         self.eager_portion_from = self.expand_from        # that way reads the step's host lists
-        self.heads = PagedSoftmax(self.H, self.H, self.dk, self.dv, float(p["scale"]))
-        self.uk_rows = self.uk.view(self.H * self.dk, self.rank)
-        self.uv_rows = self.uv_t.transpose(1, 2).view(self.H * self.dv, self.rank)
+        self.heads = PagedSoftmax(H, H, self.dq, dv, float(p["scale"]), sink=self.sink)
+        self.uk_rows = self.uk.view(H * self.dq, row)
+        self.uv_rows = self.uv_t.transpose(1, 2).view(H * dv, row)
         K.stream_lib()
 
     def cache_need(self) -> CacheNeed:
-        return CacheNeed(kv=KVNeed(1, self.rank, None, 0))       # one pool: the latents are keys and values
+        return CacheNeed(kv=KVNeed(1, self.row, None, 0))       # one pool: the latents are keys and values
+
+    def _queries(self, x, proj, ctx, cache: LayerCache) -> torch.Tensor:
+        """The queries [T, H * (dk + dr)] in the compute type, rotated where they have rotated channels; a layer that
+        makes its own latents also puts them into the pages here: normed, their rotated part turned."""
+        T, H = x.shape[0], self.H
+        direct = self.q_rank is None
+        if self.own and not (direct and self.dr):
+            K.qk_norm_rope_store(proj, ctx.positions, cache.slot_mapping, None, self.dkv_norm, self.eps, self.freq, self.amplitude,
+                                 None, cache.kpool, cache.vpool, 0, col=self.latent_col, per_head=True, adjacent=self.adjacent,
+                                 rot_at_k=self.rank, k_normed=self.rank)
+        if not direct:
+            q = K.rmsnorm_cols(proj, 0, self.dq_norm, self.eps, self.rt.dtype)
+            if not self.dr:
+                return K.linear(q, self.w_uq)
+            proj = K.linear(q, self.w_uq, out_dtype=torch.float32)
+        q = torch.empty(T, H * self.dq, dtype=self.rt.dtype, device=x.device)
+        if direct and self.own and self.dr:
+            # queries and latents lie side by side in the product's rows: one pass turns both and stores the latents
+            K.qk_norm_rope_store(proj, ctx.positions, cache.slot_mapping, None, self.dkv_norm, self.eps, self.freq, self.amplitude,
+                                 q, cache.kpool, cache.vpool, H, per_head=True, adjacent=self.adjacent, q_dim=self.dq,
+                                 rot_at_q=self.dk, rot_at_k=self.rank, k_normed=self.rank)
+        else:
+            K.qk_norm_rope_store(proj, ctx.positions, None, None, None, self.eps, self.freq, self.amplitude, q, None, None, H,
+                                 adjacent=self.adjacent, q_dim=self.dq, rot_at_q=self.dk, queries_only=True)
+        return q
+
+    def _gated(self, y, proj):
+        return K.gate_rows(y, proj, self.gate_col, every=self.dv if self.gate_per_head else 1)
 
     def forward(self, x, ctx, cache: LayerCache, out: Optional[torch.Tensor] = None):
         T, H = x.shape[0], self.H
         if cache.writes != self.own:
             raise K.KernelError("a latent_attention part writes the latents it makes, and only those")
         proj = K.linear(x, self.w_in, out_dtype=torch.float32)
-        if self.own:
-            K.qk_norm_rope_store(proj, ctx.positions, cache.slot_mapping, None, self.dkv_norm, self.eps, None, 1.0, None,
-                                 cache.kpool, cache.vpool, 0, col=self.latent_col)
-        q = K.linear(K.rmsnorm_cols(proj, 0, self.dq_norm, self.eps, self.rt.dtype), self.w_uq)
+        q = self._queries(x, proj, ctx, cache)
         if self.expand_from is not None and not ctx.recording and ctx.max_q_len >= self.expand_from:
-            y = K.gate_rows(self._over_heads(q, ctx, cache), proj, self.gate_col)
-            return K.linear(y, self.w_o, out_dtype=torch.float32, out=out)
-        # the queries as the latents see them, [T, H * rank]: a product per head, read and written in place
-        seen = torch.empty(T, H * self.rank, dtype=self.rt.dtype, device=x.device)
-        torch.bmm(q.view(T, H, self.dk).transpose(0, 1), self.uk, out=seen.view(T, H, self.rank).transpose(0, 1))
+            return K.linear(self._gated(self._over_heads(q, ctx, cache), proj), self.w_o, out_dtype=torch.float32, out=out)
+        # the queries as the rows of the pages see them, [T, H * row]: a product per head, read and written in place
+        seen = torch.empty(T, H * self.row, dtype=self.rt.dtype, device=x.device)
+        torch.bmm(q.view(T, H, self.dq).transpose(0, 1), self.uk, out=seen.view(T, H, self.row).transpose(0, 1))
         K.note_library_call()
         mixed = self.core(seen, ctx, cache.kpool, cache.kpool, cache.block_table, self.window)
-        per_head = mixed.view(T, H, self.rank).transpose(0, 1)
+        per_head = mixed.view(T, H, self.row).transpose(0, 1)
         heads = torch.bmm(per_head, self.uv_t) if mixed.dtype == torch.float32 else torch.bmm(per_head, self.uv_t, out_dtype=torch.float32)
         K.note_library_call()
-        y = K.gate_heads(heads, proj, self.gate_col, self.rt.dtype)
+        y = K.gate_heads(heads, proj, self.gate_col, self.rt.dtype, per_head=self.gate_per_head)
         return K.linear(y, self.w_o, out_dtype=torch.float32, out=out)
-
 
     def _over_heads(self, q, ctx, cache: LayerCache) -> torch.Tensor:
         """Attention with keys and values of every head written out: the pages that hold a key some token of the step
-        can see are picked out of the pool, ``k = W_uk c`` and ``v = W_uv c`` are two products over them, laid out as
-        pools of H heads, and the kernels walk them through a block table of their own that holds nothing else.  A
-        tile of queries starts at the tile of 64 keys in which its first token's window starts; the picked pages
-        start there."""
+        can see are picked out of the pool, ``k = W_uk c`` (beside the rotated channels, the same for every head) and
+        ``v = W_uv c`` are two products over them, laid out as pools of H heads, and the kernels walk them through a
+        block table of their own that holds nothing else.  A tile of queries starts at the tile of 64 keys in which its
+        first token's window starts; the picked pages start there."""
         ps, window = int(cache.kpool.shape[2]), self.window
         B, width = cache.block_table.shape
         pairs, table, at = [], np.full((B, width), -1, dtype=np.int32), 0
@@ -197,8 +268,8 @@ class LatentAttention(Part):
         flat = np.concatenate([np.concatenate(pairs).reshape(-1), table.reshape(-1)])
         dev = ctx.upload_ints(flat)
         pairs_dev, table_dev = dev[: 2 * at].view(at, 2), dev[2 * at:].view(B, width)
-        latents = K.gather_pages(cache.kpool, cache.block_table, pairs_dev).view(at * ps, self.rank)
-        keys = K.rows_to_pages(K.linear(latents, self.uk_rows), ps, self.H, self.dk)
+        latents = K.gather_pages(cache.kpool, cache.block_table, pairs_dev).view(at * ps, self.row)
+        keys = K.rows_to_pages(K.linear(latents, self.uk_rows), ps, self.H, self.dq)
         values = K.rows_to_pages(K.linear(latents, self.uv_rows), ps, self.H, self.dv)
         return self.heads(q, ctx, keys, values, table_dev, window)
 

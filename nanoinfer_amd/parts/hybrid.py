@@ -44,9 +44,10 @@ def _padded_cols(w: torch.Tensor, cols: int) -> torch.Tensor:
 
 @register_part("embedding", "scaled_table")
 class ScaledTableEmbedding(Part):
-    """``h[t] = E[id[t]] * scale + P[position[t]]``; the position rows are learned and not scaled.
-    params: vocab_size, hidden_size, scale, max_positions.  weights: weight [vocab, hidden], positions
-    [max_positions, hidden] (absent from the spec's weights: no position rows)."""
+    """``h[t] = E[id[t]] * scale + P[position[t]]``; the position rows are learned and not scaled.  With a ``norm``
+    among the weights the row is then divided by its root mean square and multiplied by that weight, in float32.
+    params: vocab_size, hidden_size, scale, max_positions, eps (of the norm).  weights: weight [vocab, hidden], positions
+    [max_positions, hidden] (absent from the spec's weights: no position rows), norm [hidden] (absent: no norm)."""
 
     graph_safe = True
 
@@ -56,6 +57,8 @@ class ScaledTableEmbedding(Part):
         out = [WeightRequest(w["weight"], (p["vocab_size"], p["hidden_size"]))]
         if "positions" in w:
             out.append(WeightRequest(w["positions"], (p["max_positions"], p["hidden_size"])))
+        if "norm" in w:
+            out.append(WeightRequest(w["norm"], (p["hidden_size"],)))
         return out
 
     def __init__(self, spec, weights, rt):
@@ -64,10 +67,13 @@ class ScaledTableEmbedding(Part):
         self.scale = float(spec.params.get("scale", 1.0))
         self.weight = rt.matrix(spec.weights["weight"], weights["weight"])
         self.positions = rt.matrix(spec.weights["positions"], weights["positions"]) if "positions" in spec.weights else None
+        self.norm = rt.vector32(spec.weights["norm"], weights["norm"]) if "norm" in spec.weights else None
+        self.eps = float(spec.params.get("eps", 0.0))
 
     def forward(self, token_ids: torch.Tensor, ctx=None) -> torch.Tensor:
         out = torch.empty(token_ids.shape[0], self.hidden_size, dtype=torch.float32, device=self.rt.device)
-        return K.embed_scaled(token_ids, ctx.positions, self.weight, self.positions, self.scale, out)
+        K.embed_scaled(token_ids, ctx.positions, self.weight, self.positions, self.scale, out)
+        return out if self.norm is None else K.post_norm(out, None, 1.0, self.norm, self.eps)
 
 
 # ------------------------------------------------------------------ what a pass adds on entering
@@ -162,15 +168,17 @@ def distance_rows(rows: int, far: float, distances: int) -> np.ndarray:
 class PagedSoftmax:
     """Causal softmax attention of ``H`` query heads on ``G`` key/value heads over pages, as the kernels of
     ``csrc/bias_attention.hip`` compute it: ``score = q . k * scale * temp(i) + bias[i - j, head]``, scores, weights and
-    both products in float32.  Holds the sizes, the constants and the kernels' tile sizes; a mixer calls it with its
-    queries and the pools it reads (keys and values may be the same pool)."""
+    both products in float32.  ``sink`` (float32 [H] on the device, or None): one more term ``exp(sink[head])`` in the
+    denominator of every row of that head, with no key and no value.  Holds the sizes, the constants and the kernels' tile
+    sizes; a mixer calls it with its queries and the pools it reads (keys and values may be the same pool)."""
 
     def __init__(self, H: int, G: int, dk: int, dv: int, scale: float, temp_coef: float = 0.0, temp_every: int = 0,
-                 bias: Optional[torch.Tensor] = None, one_pool: bool = False):
+                 bias: Optional[torch.Tensor] = None, one_pool: bool = False, sink: Optional[torch.Tensor] = None):
         if H % G:
             raise ValueError(f"{H} query heads do not divide into {G} kv heads")
         self.H, self.G, self.dk, self.dv = H, G, dk, dv
         self.scale, self.temp_coef, self.temp_every, self.bias = float(scale), float(temp_coef), int(temp_every), bias
+        self.sink = sink
         group = H // G
         self.heads_per_chunk = min(group, K.bias_attention_rows())
         self.tile_tokens = max(1, K.bias_attention_rows() // self.heads_per_chunk)
@@ -189,7 +197,8 @@ class PagedSoftmax:
             if tiles is None:
                 raise K.KernelError("this step was recorded without the tiles of its tokens")
             return K.bias_attention_mfma(qkv, kpool, vpool, block_table, tiles, ctx.positions, self.bias, out, self.H,
-                                         self.scale, self.temp_coef, self.temp_every, self.wide_heads, window, keep_first, out_scale)
+                                         self.scale, self.temp_coef, self.temp_every, self.wide_heads, window, keep_first, out_scale,
+                                         sink=self.sink)
         tiles = ctx.q_tiles(self.tile_tokens)
         if tiles is None:
             raise K.KernelError("this step was recorded without the tiles of its tokens")
@@ -205,7 +214,7 @@ class PagedSoftmax:
         ws = ctx.workspace(T * self.H * runs * (self.dv + 2)) if runs > 1 else None
         return K.bias_attention(qkv, kpool, vpool, block_table, tiles, ctx.positions, self.bias, out, self.H,
                                 self.scale, self.temp_coef, self.temp_every, self.heads_per_chunk, runs, ws, waves, window,
-                                keep_first, out_scale)
+                                keep_first, out_scale, sink=self.sink)
 
 
 @register_part("mixer", "bias_attention")
@@ -371,12 +380,17 @@ class RoutedExperts(Part):
     ``W_r x`` (float32), and optionally one more (``shared``) that every token uses with weight 1.
 
     params: hidden_size, expert_size, experts, top;
-    activation: "relu2" (an expert is ``W_down relu(W_up x)^2``) or "swiglu" (``W_down (silu(W_gate x) * (W_up x))``);
-    mix: "softmax_chosen" (the softmax over the chosen logits alone, the default) or "softmax_all" (the softmax over all
-    experts, the chosen ones' shares not renormalised); groups, keep (default 1, 1): the experts form ``groups`` equal
-    groups of neighbours, a group counts as much as its best expert, and only the best ``keep`` groups can be chosen from;
+    activation: "relu2" (an expert is ``W_down relu(W_up x)^2``), "swiglu" (``W_down (silu(W_gate x) * (W_up x))``) or
+    "capped_glu" (``g = min(W_gate x, limit)``, ``u = clamp(W_up x, -limit, limit)``, ``W_down (g sigmoid(slope g) (u + 1))``,
+    with the params ``limit`` and ``slope``);
+    mix: "softmax_chosen" (the softmax over the chosen logits alone, the default), "softmax_all" (the softmax over all
+    experts, the chosen ones' shares not renormalised) or "sigmoid" (an expert's score is the sigmoid of its logit, and the
+    chosen ones' scores are their weights as they are); mix_scale (default 1) multiplies every weight;
+    groups, keep (default 1, 1): the experts form ``groups`` equal groups of neighbours, a group counts as much as the
+    sum of its ``group_top`` (default 1) best experts, and only the best ``keep`` groups can be chosen from;
     shared: None or the PartSpec of a feed-forward.
-    weights: router [experts, d], up<e> [expert_size, d], down<e> [d, expert_size], with "swiglu" also gate<e>.
+    weights: router [experts, d], up<e> [expert_size, d], down<e> [d, expert_size], with a gated activation also gate<e>;
+    correction [experts] (absent: none): added to the scores that choose the experts and the groups, never to the weights.
 
     The experts' matrices are laid side by side, up [E * ff, d] (gated: [E * 2 ff, d], an expert's gate rows and then
     its up rows) and down [d, E * ff].  For a few rows only the chosen experts' rows are read; for many, all experts
@@ -391,8 +405,10 @@ class RoutedExperts(Part):
         p, w = spec.params, spec.weights
         d, ff = p["hidden_size"], p["expert_size"]
         out = [WeightRequest(w["router"], (p["experts"], d))]
+        if "correction" in w:
+            out.append(WeightRequest(w["correction"], (p["experts"],)))
         for e in range(p["experts"]):
-            if p.get("activation", "relu2") == "swiglu":
+            if p.get("activation", "relu2") != "relu2":
                 out.append(WeightRequest(w[f"gate{e}"], (ff, d)))
             out += [WeightRequest(w[f"up{e}"], (ff, d)), WeightRequest(w[f"down{e}"], (d, ff))]
         if p.get("shared") is not None:
@@ -405,14 +421,19 @@ class RoutedExperts(Part):
         p, names = spec.params, spec.weights
         self.E, self.top, self.ff = int(p["experts"]), int(p["top"]), int(p["expert_size"])
         activation = p.get("activation", "relu2")
-        if activation not in ("relu2", "swiglu"):
-            raise ValueError(f"expert activation {activation!r} is not known (known: 'relu2', 'swiglu')")
-        self.gated = activation == "swiglu"
-        mix = p.get("mix", "softmax_chosen")
-        if mix not in ("softmax_chosen", "softmax_all"):
-            raise ValueError(f"expert mix {mix!r} is not known (known: 'softmax_chosen', 'softmax_all')")
-        self.over_all = mix == "softmax_all"
-        self.groups, self.keep = int(p.get("groups", 1)), int(p.get("keep", 1))
+        if activation not in K.EXPERT_FORMS:
+            raise ValueError(f"expert activation {activation!r} is not known (known: {sorted(K.EXPERT_FORMS)})")
+        self.activation = activation
+        self.gated = activation != "relu2"
+        self.limit, self.slope = float(p.get("limit", 0.0)), float(p.get("slope", 1.0))
+        if activation == "capped_glu" and not self.limit > 0:
+            raise ValueError("capped experts need a positive limit")
+        self.mix = p.get("mix", "softmax_chosen")
+        if self.mix not in K.ROUTE_SCORINGS:
+            raise ValueError(f"expert mix {self.mix!r} is not known (known: {sorted(K.ROUTE_SCORINGS)})")
+        self.mix_scale = float(p.get("mix_scale", 1.0))
+        self.groups, self.keep, self.group_top = int(p.get("groups", 1)), int(p.get("keep", 1)), int(p.get("group_top", 1))
+        self.correction = rt.vector32(names["correction"], weights["correction"]) if "correction" in names else None
         if self.groups < 1 or self.E % self.groups or not 1 <= self.keep <= self.groups or self.top > self.E // self.groups * self.keep:
             raise ValueError(f"{self.top} experts cannot be chosen from {self.keep} of {self.groups} groups of {self.E}")
         self.w_router = rt.weight(names["router"], weights["router"])
@@ -428,14 +449,16 @@ class RoutedExperts(Part):
         T = x.shape[0]
         z = K.linear(x, self.w_router, out_dtype=torch.float32)
         few = T <= K.EXPERTS_FEW_ROWS
-        chosen, mix, mix_all = K.route_top(z, self.top, mix_all=not few, over_all=self.over_all, groups=self.groups, keep=self.keep)
+        chosen, mix, mix_all = K.route_top(z, self.top, mix_all=not few, groups=self.groups, keep=self.keep, scoring=self.mix,
+                                           correction=self.correction, group_top=self.group_top, scale=self.mix_scale)
         out = None
         if self.shared is not None:
             out = torch.empty(2, T, self.w_down.shape[0], dtype=torch.float32, device=x.device)
         if few:
-            y = K.experts_few(x, self.w_up.rows, self.w_down.rows, chosen, mix, self.ff, self.gated, None if out is None else out[0])
+            y = K.experts_few(x, self.w_up.rows, self.w_down.rows, chosen, mix, self.ff, self.activation, None if out is None else out[0],
+                              limit=self.limit, slope=self.slope)
         else:
-            act = K.experts_act(K.linear(x, self.w_up), mix_all, self.ff, self.gated)
+            act = K.experts_act(K.linear(x, self.w_up), mix_all, self.ff, self.activation, self.limit, self.slope)
             y = K.linear(act, self.w_down, out_dtype=torch.float32, out=None if out is None else out[0])
         if out is None:
             return y

@@ -147,9 +147,12 @@ def expert(h: np.ndarray, w: Dict[str, np.ndarray], pre: str, limit: float) -> n
     return (g * sigmoid(GLU_SLOPE * g) * (u + 1.0)) @ w[pre + "down"].T
 
 
-def route(h: np.ndarray, mlp: dict, w: Dict[str, np.ndarray], pre: str):
+def route(h: np.ndarray, mlp: dict, w: Dict[str, np.ndarray], pre: str, margins: Optional[np.ndarray] = None):
     """(chosen [T, top], weights [T, top]).  Experts are chosen by sigmoid(z) + correction, within the ``keep`` groups
-    whose two best such scores sum highest; the weights are sigmoid(z) alone, times ``scale``."""
+    whose two best such scores sum highest; the weights are sigmoid(z) alone, times ``scale``.  ``margins`` [T], if
+    given, is lowered to the smallest gap by which a token's choice was made here (between the last group kept and the
+    first one left out, and between the last expert chosen and the first one left out): a choice made by less than
+    rounding moves the scores may fall the other way in an implementation that rounds."""
     r = mlp["router"]
     E, top = r["experts"], r["top"]
     s = sigmoid(h @ w[pre + "mlp.router"].T)
@@ -160,16 +163,23 @@ def route(h: np.ndarray, mlp: dict, w: Dict[str, np.ndarray], pre: str):
     for t in range(h.shape[0]):
         by_group = choice[t].reshape(groups["count"], per)
         group_score = np.sort(by_group, axis=1)[:, -2:].sum(axis=1)
-        kept = np.argsort(-group_score, kind="stable")[: groups["keep"]]
+        ranked = np.argsort(-group_score, kind="stable")
+        kept = ranked[: groups["keep"]]
         allowed = np.full(E, -np.inf)
         for g in kept:
             allowed[g * per:(g + 1) * per] = choice[t, g * per:(g + 1) * per]
-        chosen[t] = np.argsort(-allowed, kind="stable")[:top]
+        order = np.argsort(-allowed, kind="stable")
+        chosen[t] = order[:top]
+        if margins is not None:
+            if groups["keep"] < groups["count"]:
+                margins[t] = min(margins[t], group_score[ranked[groups["keep"] - 1]] - group_score[ranked[groups["keep"]]])
+            if top < E and np.isfinite(allowed[order[top]]):
+                margins[t] = min(margins[t], allowed[order[top - 1]] - allowed[order[top]])
     return chosen, np.take_along_axis(s, chosen, axis=1) * r["scale"]
 
 
-def feed_forward(h: np.ndarray, mlp: dict, w: Dict[str, np.ndarray], pre: str) -> np.ndarray:
-    chosen, weights = route(h, mlp, w, pre)
+def feed_forward(h: np.ndarray, mlp: dict, w: Dict[str, np.ndarray], pre: str, margins: Optional[np.ndarray] = None) -> np.ndarray:
+    chosen, weights = route(h, mlp, w, pre, margins)
     out = np.zeros((h.shape[0], w[pre + "mlp.e0.down"].shape[0]), dtype=F)
     for t in range(h.shape[0]):
         for e, a in zip(chosen[t], weights[t]):
@@ -181,8 +191,10 @@ def feed_forward(h: np.ndarray, mlp: dict, w: Dict[str, np.ndarray], pre: str) -
 
 # ------------------------------------------------------------------ the model
 
-def forward(cfg: dict, w: Dict[str, np.ndarray], tokens: List[int], layers_out: Optional[list] = None) -> np.ndarray:
-    """Logits [T, vocab] of one whole sequence.  ``layers_out``, if a list, gets the stream behind every layer."""
+def forward(cfg: dict, w: Dict[str, np.ndarray], tokens: List[int], layers_out: Optional[list] = None,
+            margins: Optional[np.ndarray] = None) -> np.ndarray:
+    """Logits [T, vocab] of one whole sequence.  ``layers_out``, if a list, gets the stream behind every layer;
+    ``margins`` [T] (start it at infinity) the smallest gap by which any router chose for each token (see ``route``)."""
     eps, alpha = cfg["norm"]["eps"], cfg["postln_alpha"]
     w = {k: np.asarray(v, dtype=F) for k, v in w.items()}
     x = embed(tokens, cfg, w)
@@ -199,7 +211,7 @@ def forward(cfg: dict, w: Dict[str, np.ndarray], tokens: List[int], layers_out: 
             raise ValueError(f"layer type {layer['type']!r}")
         x = rms(alpha * x + y, eps) * w[pre + "norm1"]
         if layer.get("mlp") is not None:
-            x = rms(alpha * x + feed_forward(x, layer["mlp"], w, pre), eps) * w[pre + "norm2"]
+            x = rms(alpha * x + feed_forward(x, layer["mlp"], w, pre, margins), eps) * w[pre + "norm2"]
         if layers_out is not None:
             layers_out.append(x)
     return (rms(x, eps) * w["final.norm"]) @ w["head"].T

@@ -453,17 +453,45 @@ def ruludra_config(layers: int, vocab: int, like: dict) -> dict:
             "logit_scale": float(width) ** -0.5, "layers": out}
 
 
+def vimilix_config(layers: int, vocab: int, like: dict) -> dict:
+    """A Vimilix model whose layers have the sizes of a Llama shape's, four kinds in turn: attention over a latent of 192
+    numbers a token beside 64 rotated key channels that the heads share (the shape's heads, 64 + 64 channels a query head,
+    values of the shape's head size), attention in a window of 1,024 with a sink (the shape's heads and head size, half of
+    every head rotated and stretched), a second latent layer, and a second windowed layer that reads the keys and values
+    of the first; every layer with the routed experts of the Fusavik shape (sixteen of an eighth of the shape's
+    feed-forward of which a token uses four, out of two of four groups, and a shared expert of a quarter of it), capped."""
+    width, ff, hd = like["hidden_size"], like["intermediate_size"], like["head_dim"]
+    heads = like["num_attention_heads"]
+    latent = {"type": "latent_attention", "mixer": {"heads": heads, "dim": 64, "rot_dim": 64, "vdim": hd, "kv_rank": 192,
+                                                    "scale": 128 ** -0.5, "rot": {"base": 50000.0, "dims": 64}}}
+    window = {"heads": heads, "kv_heads": like["num_key_value_heads"], "dim": hd, "vdim": hd, "scale": hd ** -0.5, "mask": {"size": 1024},
+              "rot": {"base": 500000.0, "dims": hd // 2, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 2048}}}
+    routed = {"kind": "moe", "expert": {"ff": ff // 8, "limit": 7.0},
+              "router": {"experts": 16, "top": 4, "scale": 1.5, "groups": {"count": 4, "keep": 2}}, "shared": {"ff": ff // 4, "limit": 7.0}}
+    out = []
+    for i in range(layers):
+        if i % 2 == 0:
+            out.append(dict(latent, mlp=routed))
+        elif i % 4 == 1:
+            out.append({"type": "attention", "mixer": dict(window), "mlp": routed})
+        else:
+            out.append({"type": "attention", "mixer": dict(window, kv_from=i - 2), "mlp": routed})
+    return {"architecture": "Vimilix", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "postln_alpha": 2.0, "layers": out}
+
+
 def hybrid(args) -> int:
     """``--workload hybrid``: prefill of one prompt and decode steps of the Zekalorn shape above and of the Llama
     shape of equal depth, one JSON line with both.  ``--workload stateful``: the same of the Fusavik shape above
     beside the Zekalorn shape (the framework's other model with mixers that keep a state and routed experts).
     ``--workload latent``: the same of the Ruludra shape above beside the Fusavik shape (the framework's other model
-    with attention in a window, a matrix memory a head and a pair-hash embedding)."""
+    with attention in a window, a matrix memory a head and a pair-hash embedding).  ``--workload postnorm``: the same of
+    the Vimilix shape above beside the Fusavik shape (the framework's other model with attention in a window and routed
+    experts chosen within groups beside a shared one)."""
     import torch
     torch.cuda.set_device(0)
     layers = args.layers or 8
     prompt, batch = args.prompt_len, args.batch
-    first = {"stateful": "fusavik", "latent": "ruludra"}.get(args.workload, "zekalorn")
+    first = {"stateful": "fusavik", "latent": "ruludra", "postnorm": "vimilix"}.get(args.workload, "zekalorn")
     out = {"metric": f"{args.workload}_decode_tokens_per_s", "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
            "higher_is_better": True, "dtype": args.dtype, "data": "synthetic token ids, random-init weights",
            "config": {"layers": layers, "prompt_len": prompt, "global_batch": batch, "shape": args.shape,
@@ -475,6 +503,8 @@ def hybrid(args) -> int:
         shapes = {"fusavik": fusavik_config(layers, 128256, like), "zekalorn": shapes["zekalorn"]}
     if args.workload == "latent":
         shapes = {"ruludra": ruludra_config(layers, 128256, like), "fusavik": fusavik_config(layers, 128256, like)}
+    if args.workload == "postnorm":
+        shapes = {"vimilix": vimilix_config(layers, 128256, like), "fusavik": fusavik_config(layers, 128256, like)}
     for name, cfg in shapes.items():
         if args.only and name != args.only:
             continue
@@ -531,14 +561,15 @@ def main() -> int:
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64 and the further points")
     ap.add_argument("--no-further", action="store_true",
                     help="skip the points beyond the default line's: contexts of 8k and 32k, float32, the 3B shape")
-    ap.add_argument("--only", default=None, choices=["zekalorn", "llama", "fusavik", "ruludra"],
-                    help="hybrid, stateful, latent: measure one of the two models")
-    ap.add_argument("--workload", default="steps", choices=["steps", "serving", "hybrid", "stateful", "latent"],
+    ap.add_argument("--only", default=None, choices=["zekalorn", "llama", "fusavik", "ruludra", "vimilix"],
+                    help="hybrid, stateful, latent, postnorm: measure one of the two models")
+    ap.add_argument("--workload", default="steps", choices=["steps", "serving", "hybrid", "stateful", "latent", "postnorm"],
                     help="steps: the decode step and prefill of the result line's contract (default); "
                          "serving: concurrent requests through the engine's scheduler, a line of its own; "
                          "hybrid: prefill and decode of a Zekalorn model at the 1B shape's layer sizes beside the Llama shape; "
                          "stateful: the same of a Fusavik model beside the Zekalorn one; "
-                         "latent: the same of a Ruludra model beside the Fusavik one")
+                         "latent: the same of a Ruludra model beside the Fusavik one; "
+                         "postnorm: the same of a Vimilix model beside the Fusavik one")
     ap.add_argument("--requests", type=int, default=64, help="serving: concurrent requests")
     ap.add_argument("--new-tokens", type=int, default=256, help="serving: tokens generated per request")
     ap.add_argument("--min-prompt", type=int, default=128, help="serving: shortest prompt")
@@ -559,7 +590,7 @@ def main() -> int:
         return 2
     if args.workload == "serving":
         return serving(args)
-    if args.workload in ("hybrid", "stateful", "latent"):
+    if args.workload in ("hybrid", "stateful", "latent", "postnorm"):
         return hybrid(args)
     args.prefill_chunk = args.prefill_chunk or PREFILL_CHUNK
 

@@ -655,15 +655,16 @@ bias_attention_mfma_kernel(const T* __restrict__ qkv, int row_stride, const T* _
 
 // out[row, :] = sum_r acc_r e^(m_r - M) / (sum_r l_r e^(m_r - M) + e^(sink - M)) over the runs of a row (an empty run
 // has l = 0; no sink: no such term; M is the maximum over the runs and the sink).
-// One wavefront a row; lane r takes run r's maximum and sum (n_runs <= 64), the weights e^(m_r - M) go through LDS,
-// and the sums over the runs then read nothing that depends on an earlier read.
+// The weights e^(m_r - M) go through LDS, and the sums over the runs then read nothing that depends on an earlier read.
+// One workgroup a row, of as many wavefronts as the row has runs of 64 value channels (up to four); every wavefront works
+// the runs' weights out for itself (lane r takes run r's maximum and sum, n_runs <= 64) and sums its own channels.
 template <typename T>
-__global__ void __launch_bounds__(WAVE) merge_runs_kernel(const float* __restrict__ partial, T* __restrict__ out, int n_runs, int dv,
-                                                          float out_scale, const float* __restrict__ sink, int H) {
-    __shared__ float weight[WAVE];
+__global__ void __launch_bounds__(MAX_VCHUNKS * WAVE) merge_runs_kernel(const float* __restrict__ partial, T* __restrict__ out, int n_runs,
+                                                                        int dv, float out_scale, const float* __restrict__ sink, int H) {
+    __shared__ float weight[MAX_VCHUNKS][WAVE];
     const size_t row = blockIdx.x;
     const float* p = partial + row * n_runs * (dv + 2);
-    const int lane = threadIdx.x;
+    const int lane = threadIdx.x & (WAVE - 1), wave = threadIdx.x / WAVE;
     float m = -INFINITY, l = 0.f;
     if (lane < n_runs) {
         m = p[lane * (dv + 2)];
@@ -675,12 +676,12 @@ __global__ void __launch_bounds__(WAVE) merge_runs_kernel(const float* __restric
     M = fmaxf(M, sk);
     const float w = l > 0.f ? expf(m - M) : 0.f;
     const float L = wave_sum(l * w) + (sink ? expf(sk - M) : 0.f);
-    weight[lane] = w;
-    __syncthreads();
-    for (int c = lane; c < dv; c += WAVE) {
+    weight[wave][lane] = w;
+    __builtin_amdgcn_wave_barrier();          // a wavefront reads only the weights it wrote itself
+    for (int c = wave * WAVE + lane; c < dv; c += blockDim.x) {
         float a = 0.f;
         for (int r = 0; r < n_runs; ++r) {
-            const float wr = weight[r];
+            const float wr = weight[wave][r];
             if (wr > 0.f) a += p[r * (dv + 2) + 2 + c] * wr;
         }
         st(out + row * dv + c, a * out_scale / L);
@@ -731,7 +732,7 @@ NI_EXPORT int ni_bias_attention(const void* qkv, int row_stride, const void* kpo
             (const int32_t*)tiles, (const int32_t*)positions, (const float*)bias, distances, (float*)out, H, G, dk, dv, page_size, scale, temp_coef,
             temp_every, heads_per_chunk, n_runs, (float*)partial, k_pieces, v_pieces, dkp, window, keep_first, out_scale,
             (const float*)sink);
-        if (partial) merge_runs_kernel<float><<<n_rows * H, 64, 0, stream>>>((const float*)partial, (float*)out, n_runs, dv, out_scale,
+        if (partial) merge_runs_kernel<float><<<n_rows * H, std::min(MAX_VCHUNKS, (dv + WAVE - 1) / WAVE) * WAVE, 0, stream>>>((const float*)partial, (float*)out, n_runs, dv, out_scale,
                                                                              (const float*)sink, H);
     } else {
         static size_t allowed = 48 * 1024;
@@ -743,7 +744,7 @@ NI_EXPORT int ni_bias_attention(const void* qkv, int row_stride, const void* kpo
             (const int32_t*)tiles, (const int32_t*)positions, (const float*)bias, distances, (bf16_t*)out, H, G, dk, dv, page_size, scale, temp_coef,
             temp_every, heads_per_chunk, n_runs, (float*)partial, k_pieces, v_pieces, dkp, window, keep_first, out_scale,
             (const float*)sink);
-        if (partial) merge_runs_kernel<bf16_t><<<n_rows * H, 64, 0, stream>>>((const float*)partial, (bf16_t*)out, n_runs, dv, out_scale,
+        if (partial) merge_runs_kernel<bf16_t><<<n_rows * H, std::min(MAX_VCHUNKS, (dv + WAVE - 1) / WAVE) * WAVE, 0, stream>>>((const float*)partial, (bf16_t*)out, n_runs, dv, out_scale,
                                                                               (const float*)sink, H);
     }
     return NI_LAUNCH_RESULT();

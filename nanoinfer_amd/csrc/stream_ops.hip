@@ -245,12 +245,43 @@ NI_EXPORT int ni_add_rmsnormed(void* h, const void* y, const void* w, int T, int
 // The stream itself takes the normed sum (a block whose norm stands behind the sum); x, if given, is the same in the
 // compute type for the products that read it next.  addends float32 [n_addends][T][d], summed in their order and then
 // added to alpha * h; all of it float32.  A thread reads in the second pass what it wrote itself in the first.
+#define POST_NORM_ITEMS 8       // elements of a row a thread keeps in registers: rows of up to 8 * 512 elements
+
 template <typename X>
 __global__ void post_norm_kernel(float* __restrict__ h, const float* __restrict__ addends, int n_addends, size_t addend_stride,
                                  float alpha, const float* __restrict__ w, float eps, X* __restrict__ x, int d) {
     __shared__ float scratch[16];
     const size_t base = static_cast<size_t>(blockIdx.x) * d;
     float ss = 0.f;
+    if (d <= POST_NORM_ITEMS * static_cast<int>(blockDim.x)) {
+        // the row stays in registers between the sum and the division: every element is read once and written once
+        float v[POST_NORM_ITEMS];
+#pragma unroll
+        for (int u = 0; u < POST_NORM_ITEMS; ++u) {
+            const int i = threadIdx.x + u * blockDim.x;
+            v[u] = 0.f;
+            if (i < d) {
+                v[u] = alpha * h[base + i];
+                if (n_addends > 0) {
+                    float a = addends[base + i];
+                    for (int s = 1; s < n_addends; ++s) a += addends[s * addend_stride + base + i];
+                    v[u] += a;
+                }
+                ss += v[u] * v[u];
+            }
+        }
+        const float inv = 1.0f / sqrtf(block_sum(ss, scratch) / static_cast<float>(d) + eps);
+#pragma unroll
+        for (int u = 0; u < POST_NORM_ITEMS; ++u) {
+            const int i = threadIdx.x + u * blockDim.x;
+            if (i < d) {
+                const float r = (v[u] * inv) * w[i];
+                h[base + i] = r;
+                if (x) st(x + base + i, r);
+            }
+        }
+        return;
+    }
     for (int i = threadIdx.x; i < d; i += blockDim.x) {
         float v = alpha * h[base + i];
         if (n_addends > 0) {
@@ -617,6 +648,10 @@ __global__ void route_top_kernel(const float* __restrict__ z, const float* __res
         total = wave_sum(sum);
     }
     unsigned taken_mask = 0;        // bit j: this lane's expert lane + 64 j has been chosen
+    // up to 64 chosen experts stay in registers, the k-th in lane k; more go through the result's own memory
+    const bool in_lanes = top <= WAVE;
+    int my_expert = 0;
+    float my_value = -INFINITY;
     for (int k = 0; k < top; ++k) {
         float v = -INFINITY;
         int at = NO_EXPERT;
@@ -636,7 +671,25 @@ __global__ void route_top_kernel(const float* __restrict__ z, const float* __res
         for (int j = 0; j < SLOTS; ++j)
             if (lane + j * WAVE == cand) mine = raw[j];
         const float value = wave_sum(mine);
-        if (lane == 0) { c[k] = cand; m[k] = value; }
+        if (in_lanes) {
+            if (lane == k) { my_expert = cand; my_value = value; }
+        } else if (lane == 0) {
+            c[k] = cand;
+            m[k] = value;
+        }
+    }
+    if (in_lanes) {
+        if (scoring == 0) {         // the softmax among the chosen
+            best = wave_max(my_value);
+            total = wave_sum(lane < top ? expf(my_value - best) : 0.f);
+        }
+        if (lane < top) {
+            const float w = (scoring == 2 ? my_value : expf(my_value - best) / total) * route_scale;
+            c[lane] = my_expert;
+            m[lane] = w;
+            if (mix_all) mix_all[static_cast<size_t>(t) * E + my_expert] = w;
+        }
+        return;
     }
     if (lane == 0) {
         if (scoring == 0) {         // the softmax among the chosen

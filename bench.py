@@ -463,7 +463,7 @@ def vimilix_config(layers: int, vocab: int, like: dict) -> dict:
     width, ff, hd = like["hidden_size"], like["intermediate_size"], like["head_dim"]
     heads = like["num_attention_heads"]
     latent = {"type": "latent_attention", "mixer": {"heads": heads, "dim": 64, "rot_dim": 64, "vdim": hd, "kv_rank": 192,
-                                                    "scale": 128 ** -0.5, "rot": {"base": 50000.0, "dims": 64}}}
+                                                    "scale": 128 ** -0.5, "rot": {"base": 10000.0, "dims": 64}}}
     window = {"heads": heads, "kv_heads": like["num_key_value_heads"], "dim": hd, "vdim": hd, "scale": hd ** -0.5, "mask": {"size": 1024},
               "rot": {"base": 500000.0, "dims": hd // 2, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 2048}}}
     routed = {"kind": "moe", "expert": {"ff": ff // 8, "limit": 7.0},
@@ -476,7 +476,7 @@ def vimilix_config(layers: int, vocab: int, like: dict) -> dict:
             out.append({"type": "attention", "mixer": dict(window), "mlp": routed})
         else:
             out.append({"type": "attention", "mixer": dict(window, kv_from=i - 2), "mlp": routed})
-    return {"architecture": "Vimilix", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "postln_alpha": 2.0, "layers": out}
+    return {"architecture": "Vimilix", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "postln_alpha": 1.5, "layers": out}
 
 
 def hybrid(args) -> int:

@@ -78,6 +78,9 @@ class KeyedAttention(WindowAttention):
 # the longest portion of a step from which on a latent attention writes keys and values of every head out for the step
 # (None: never): below it the products over all visible latents cost more than attention over the latents themselves saves
 LATENT_EXPAND_FROM = 256
+# the most channels a token's row in the pages may have for attention over the rows themselves (the attention kernels'
+# value channels); a wider row is only ever read through the written-out way
+LATENT_ROW_MAX = 256
 
 
 @register_part("mixer", "latent_attention")
@@ -109,7 +112,8 @@ class LatentAttention(Part):
     params: hidden_size, num_heads, key_dim, value_dim, q_rank (None: the queries are ``W_q x``, no latent of their own),
     rank, scale, window (None: every earlier key), eps, rot_dim (default 0), position, adjacent_pairs, gate ("channel", the
     default: a gate a value channel; "head": one a head), expand_from (default ``LATENT_EXPAND_FROM``; None: never; it is
-    never taken where ``rank + rot_dim < key_dim + rot_dim + value_dim``).
+    never taken where ``rank + rot_dim < key_dim + rot_dim + value_dim``, and always where ``rank + rot_dim`` is more than
+    ``LATENT_ROW_MAX``: such a part reads the host lists in every step and is not ``graph_safe``).
     weights: dq [q_rank, d], dq_norm [q_rank], uq [H*(dk+r), q_rank] (or q [H*(dk+r), d]), dkv [rank + r, d] and dkv_norm
     [rank] (both or neither), uk [H*dk, rank], uv [H*dv, rank], g [H*dv, d] (or [H, d]), o [d, H*dv], sink [H] (absent:
     none; one more term ``exp(sink[h])`` in the softmax's denominator)."""
@@ -152,8 +156,11 @@ class LatentAttention(Part):
             raise ValueError(f"gate {gate!r} is not 'channel' or 'head'")
         self.gate_per_head = gate == "head"
         H, dk, dv, dr, rank, row = self.H, self.dk, self.dv, self.dr, self.rank, self.row
-        if row > 256:
-            raise ValueError(f"a latent of {rank} + {dr} channels is more than the attention kernels' 256 value channels")
+        # rows of more channels than the attention kernels take as values: every step writes the heads' keys and values
+        # out, which reads the step's host lists, so no step of such a model is recorded
+        self.always_expand = row > LATENT_ROW_MAX
+        if self.always_expand:
+            self.graph_safe = False
         self.freq, self.amplitude, self.adjacent = None, 1.0, bool(p.get("adjacent_pairs", False))
         if dr:
             from .standard import build_part
@@ -190,7 +197,7 @@ class LatentAttention(Part):
         # steps with long portions: keys and values of every head are made of the latents the step can see, once,
         # and attention runs at the heads' own sizes
         self.expand_from = p.get("expand_from", LATENT_EXPAND_FROM)
-        if row < self.dq + dv:      # attention over the latents is then the smaller sum of products already
+        if row < self.dq + dv and not self.always_expand:      # attention over the latents is then the smaller sum of products already
             self.expand_from = None
         if self.expand_from is not None:
             self.expand_from = max(2, int(self.expand_from))
@@ -237,7 +244,7 @@ class LatentAttention(Part):
             raise K.KernelError("a latent_attention part writes the latents it makes, and only those")
         proj = K.linear(x, self.w_in, out_dtype=torch.float32)
         q = self._queries(x, proj, ctx, cache)
-        if self.expand_from is not None and not ctx.recording and ctx.max_q_len >= self.expand_from:
+        if self.always_expand or (self.expand_from is not None and not ctx.recording and ctx.max_q_len >= self.expand_from):
             return K.linear(self._gated(self._over_heads(q, ctx, cache), proj), self.w_o, out_dtype=torch.float32, out=out)
         # the queries as the rows of the pages see them, [T, H * row]: a product per head, read and written in place
         seen = torch.empty(T, H * self.row, dtype=self.rt.dtype, device=x.device)

@@ -156,7 +156,7 @@ def test_zz_report_worst_rows():
 
 # ------------------------------------------------------------------ every mechanism alone
 
-ALONE = ["sink_only", "sink_open", "latent_only", "latent_odd", "moe_only", "moe_flat", "moe_singles", "shared_open"]
+ALONE = ["sink_only", "sink_open", "latent_only", "latent_odd", "latent_huge", "moe_only", "moe_flat", "moe_singles", "shared_open"]
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -178,7 +178,7 @@ def test_one_mechanism_whole_prompt_and_token_by_token(name, dtype):
 # ------------------------------------------------------------------ the whole design, every schedule
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name", ["mixed", "shared_kv", "odd_sizes"])
+@pytest.mark.parametrize("name", ["mixed", "shared_kv", "odd_sizes", "latent_huge"])
 def test_portions_of_several_sizes_down_to_two_tokens(name, dtype):
     folder = folder_of(name)
     toks = random_tokens(Z.ALL[name]["vocab"], 150, 21)

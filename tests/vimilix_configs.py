@@ -65,6 +65,8 @@ SHARED_OPEN = model(48, 50, [(sink(2, 1, 16, 16, 0.3, rot(16, 1000.0), mask=5), 
 # latents wider than a head's keys and values together: long portions write the heads' keys and values out for the step
 LATENT_WIDE = model(64, 97, [(latent(3, 8, 8, 8, 40, 0.3, mask=70), None), (latent(2, 4, 4, 12, 28, 0.4), moe(4, 2, 16, 1.0)),
                              (latent(4, 8, 16, 8, 48, 0.25, mask=5), None)])
+# a latent of more channels than the attention kernels take as values: every step writes the heads' keys and values out
+LATENT_HUGE = model(64, 97, [(latent(2, 8, 16, 8, 272, 0.3), moe(4, 2, 16, 1.0)), (latent(3, 16, 4, 8, 300, 0.25, mask=40), None)])
 # sizes that are multiples of nothing much: a width of 50, experts of 37 and 45, a vocabulary of 61
 ODD_SIZES = model(50, 61, [(sink(2, 1, 12, 10, 0.3, rot(6, 77.0), mask=11), moe(6, 2, 37, 1.1, groups=(3, 2), shared=(45, 1.7))),
                            (latent(2, 6, 2, 10, 14, 0.3, mask=17), moe(3, 3, 9, 2.0)),
@@ -74,11 +76,11 @@ MIXED = model(72, 131, [(latent(3, 16, 16, 24, 32, 0.2, base=2000.0), moe(8, 3, 
                         (sink(6, 2, 16, 24, 0.3, rot(8, 5000.0, (8.0, 1.0, 4.0, 128)), mask=33), moe(6, 2, 32, 1.0, shared=(16, 1.0))),
                         (latent(5, 8, 8, 16, 40, 0.3, mask=70), None),
                         (sink(4, 2, 16, 24, 0.25, rot(8, 5000.0, (8.0, 1.0, 4.0, 128)), mask=130, kv_from=1),
-                         moe(9, 4, 16, 2.0, scale=0.75, groups=(3, 2)))], alpha=2.0)
+                         moe(9, 4, 16, 2.0, scale=0.75, groups=(3, 2)))], alpha=1.75)
 # softmax that picks one key: whether the key at a window's edge is seen decides the output
 SHARP = model(64, 97, [(sink(4, 2, 16, 16, 6.0, rot(8, 100.0), mask=19), None), (latent(2, 16, 8, 16, 24, 5.0, mask=23), None),
                        (sink(2, 2, 16, 16, 6.0, rot(8, 100.0), mask=66, kv_from=0), None)])
 
 ALL = {"sink_only": SINK_ONLY, "sink_open": SINK_OPEN, "latent_only": LATENT_ONLY, "latent_odd": LATENT_ODD, "moe_only": MOE_ONLY,
-       "moe_flat": MOE_FLAT, "moe_singles": MOE_SINGLES, "shared_kv": SHARED_KV, "shared_open": SHARED_OPEN, "latent_wide": LATENT_WIDE,
+       "moe_flat": MOE_FLAT, "moe_singles": MOE_SINGLES, "shared_kv": SHARED_KV, "shared_open": SHARED_OPEN, "latent_wide": LATENT_WIDE, "latent_huge": LATENT_HUGE,
        "odd_sizes": ODD_SIZES, "mixed": MIXED, "sharp": SHARP}

@@ -567,8 +567,9 @@ NI_EXPORT int ni_rows_to_pages(const void* x, void* y, int n_pages, int page, in
 // equal ones) can be chosen: the others' scores count as minus infinity.
 // chosen int32 [T, top], mix float32 [T, top], and (if asked for) the same as a row over all experts, zero where
 // an expert was not chosen.
-// One wavefront a row: a lane keeps the scores of experts lane, lane + 64, ...; each round finds the
-// largest score not yet taken (the lowest index among equal ones) by two butterflies over the lanes.
+// One wavefront a row.  More than 64 experts: a lane keeps the scores of experts lane, lane + 64, ...; each round finds
+// the largest score not yet taken (the lowest index among equal ones) by two butterflies over the lanes.  Up to 64
+// experts: `route_top_lanes_kernel` below, which ranks instead of searching.
 #define NO_EXPERT 0x7fffffff
 
 __device__ __forceinline__ int lowest_of(int cand) {
@@ -706,14 +707,77 @@ __global__ void route_top_kernel(const float* __restrict__ z, const float* __res
     }
 }
 
+// The same for up to 64 experts, one a lane, without butterflies: a lane ranks its expert among the others by walking
+// the E lanes' values (each read into a scalar register, `lane_value`; a lone wavefront's time is its instructions,
+// so the walks stop at E), first inside its group (which experts count
+// for the group's score), then its group among the groups, then its expert among those that may be chosen; the
+// expert of rank k is the k-th choice.  Better is: the larger score, or of equal scores the lower index, as above.
+__device__ __forceinline__ float lane_value(float v, int j) { return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), j)); }
+__device__ __forceinline__ int lane_value(int v, int j) { return __builtin_amdgcn_readlane(v, j); }
+__device__ __forceinline__ bool better(float a, int ia, float b, int ib) { return a > b || (a == b && ia < ib); }
+
+__global__ void __launch_bounds__(WAVE)
+route_top_lanes_kernel(const float* __restrict__ z, const float* __restrict__ correction, int32_t* __restrict__ chosen,
+                       float* __restrict__ mix, float* __restrict__ mix_all, int E, int top, int scoring, int n_groups, int keep,
+                       int group_top, float route_scale) {
+    const int t = blockIdx.x, e = threadIdx.x;
+    const bool mine = e < E;
+    float ze = mine ? z[static_cast<size_t>(t) * E + e] : -INFINITY;
+    if (!(ze == ze)) ze = -INFINITY;                  // a logit that is no number is never preferred
+    const float raw = scoring == 2 ? 1.0f / (1.0f + expf(-ze)) : ze;
+    const float val = mine ? raw + (correction ? correction[e] : 0.f) : -INFINITY;
+    bool open = mine;
+    if (n_groups > 1) {
+        const int per_group = E / n_groups;
+        const int grp = mine ? e / per_group : -1;
+        int in_group = 0;                             // experts of my group that are better than mine
+        for (int j = 0; j < E; ++j)
+            in_group += (lane_value(grp, j) == grp && better(lane_value(val, j), j, val, e)) ? 1 : 0;
+        const float counted = (mine && in_group < group_top) ? val : 0.f;
+        float score = 0.f;                            // of my group: the sum of its `group_top` best scores
+        for (int j = 0; j < E; ++j)
+            score += lane_value(grp, j) == grp ? lane_value(counted, j) : 0.f;
+        const int first = (mine && e % per_group == 0) ? grp : -1;      // a group's first lane speaks for it
+        int ahead = 0;                                // groups that are better than mine
+        for (int j = 0; j < E; ++j) {
+            const int gj = lane_value(first, j);
+            ahead += (gj >= 0 && better(lane_value(score, j), gj, score, grp)) ? 1 : 0;
+        }
+        open = mine && ahead < keep;
+    }
+    const unsigned long long open_mask = __ballot(open);
+    int rank = 0;                                     // experts that may be chosen and are better than mine
+    for (int j = 0; j < E; ++j)
+        rank += (((open_mask >> j) & 1ull) && better(lane_value(val, j), j, val, e)) ? 1 : 0;
+    const bool taken = open && rank < top;
+    const unsigned long long taken_mask = __ballot(taken);
+    float w = raw;
+    if (scoring != 2) {
+        const unsigned long long over = scoring == 1 ? __ballot(mine) : taken_mask;     // what the softmax runs over
+        float best = -INFINITY, total = 0.f;
+        for (int j = 0; j < E; ++j)
+            if ((over >> j) & 1ull) best = fmaxf(best, lane_value(raw, j));
+        const float mine_exp = raw > -INFINITY ? expf(raw - best) : 0.f;
+        for (int j = 0; j < E; ++j)
+            if ((over >> j) & 1ull) total += lane_value(mine_exp, j);
+        w = mine_exp / total;
+    }
+    w *= route_scale;
+    if (taken) {
+        chosen[static_cast<size_t>(t) * top + rank] = e;
+        mix[static_cast<size_t>(t) * top + rank] = w;
+    }
+    if (mix_all && mine) mix_all[static_cast<size_t>(t) * E + e] = taken ? w : 0.f;
+}
+
 NI_EXPORT int ni_route_top(const void* z, const void* correction, void* chosen, void* mix, void* mix_all, int T, int E, int top,
                            int scoring, int n_groups, int keep, int group_top, float route_scale, hipStream_t stream) {
     if (T <= 0) return 0;
     if (top < 1 || top > E || E > 32 * WAVE || scoring < 0 || scoring > 2 || group_top < 1) return -1;
     if (n_groups < 1 || n_groups > WAVE || E % n_groups || keep < 1 || keep > n_groups || top > E / n_groups * keep) return -1;
     if (E <= WAVE)
-        route_top_kernel<1><<<T, WAVE, 0, stream>>>((const float*)z, (const float*)correction, (int32_t*)chosen, (float*)mix,
-                                                    (float*)mix_all, T, E, top, scoring, n_groups, keep, group_top, route_scale);
+        route_top_lanes_kernel<<<T, WAVE, 0, stream>>>((const float*)z, (const float*)correction, (int32_t*)chosen, (float*)mix,
+                                                       (float*)mix_all, E, top, scoring, n_groups, keep, group_top, route_scale);
     else if (E <= 4 * WAVE)
         route_top_kernel<4><<<T, WAVE, 0, stream>>>((const float*)z, (const float*)correction, (int32_t*)chosen, (float*)mix,
                                                     (float*)mix_all, T, E, top, scoring, n_groups, keep, group_top, route_scale);

@@ -69,7 +69,8 @@ class SinkAttention(WindowAttention):
         super().__init__(type(spec)(spec.kind, p, spec.weights), weights, rt)
         names = spec.weights
         self.adjacent = bool(p.get("adjacent_pairs", False))
-        self.cache_window = None if p.get("cache_window", p.get("window")) is None else int(p.get("cache_window", p.get("window")))
+        kept = p["cache_window"] if "cache_window" in p else p.get("window")      # what the pages keep; absent: this part's own window
+        self.cache_window = None if kept is None else int(kept)
         if self.cache_window is not None and (self.window is None or self.window > self.cache_window):
             raise ValueError(f"a window of {self.window} keys reads pages that keep {self.cache_window}")
         self.head_q_norm = rt.vector32(names["q_norm"], weights["q_norm"])

@@ -513,6 +513,13 @@ bias_attention_kernel(const T* __restrict__ qkv, int row_stride, const T* __rest
 #define MROWS 64
 typedef float floatx4_t __attribute__((ext_vector_type(4)));
 
+// floats of the first region of the kernel's staging memory: the queries [MROWS][dk + 4], whose place the tiles of values
+// [KEYS][dv + 4] take once the queries are in registers (no tile of values where keys and values are one pool)
+__host__ __device__ __forceinline__ size_t mfma_first_floats(int dk, int dv, bool one_pool) {
+    const size_t q = static_cast<size_t>(MROWS) * (dk + 4), v = one_pool ? 0 : static_cast<size_t>(KEYS) * (dv + 4);
+    return q > v ? q : v;
+}
+
 __device__ __forceinline__ float groups4(float x, bool take_max) {
     // over the four lanes that hold one row (lanes r, r + 16, r + 32, r + 48): maximum or sum
     const auto a = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
@@ -523,7 +530,9 @@ __device__ __forceinline__ float groups4(float x, bool take_max) {
     return take_max ? fmaxf(s, t) : s + t;
 }
 
-template <typename T>
+// QS: 16-byte pieces of a lane's quarter of a query row at most (dk <= 64 QS); DVB: blocks of 16 value channels at most
+// (dv <= 16 DVB).  Both size arrays of registers, so the kernel is compiled for a few pairs of them.
+template <typename T, int QS, int DVB>
 __global__ void __launch_bounds__(WAVES * WAVE)
 bias_attention_mfma_kernel(const T* __restrict__ qkv, int row_stride, const T* __restrict__ kpool, const T* __restrict__ vpool,
                            const int32_t* __restrict__ block_table, int table_width, const int32_t* __restrict__ tiles,
@@ -533,11 +542,13 @@ bias_attention_mfma_kernel(const T* __restrict__ qkv, int row_stride, const T* _
                            float out_scale, const float* __restrict__ sink) {
     extern __shared__ __attribute__((aligned(16))) float lds[];
     const int dkp = dk + 4, dvp = dv + 4;         // strides that spread the sixteen rows of a read over the banks
-    float* Qs = lds;                              // [MROWS][dkp]
-    float* Ks = Qs + MROWS * dkp;                 // [KEYS][dkp]
     // keys and values that are one pool (dv = dk) are staged once: the values are read from the keys' tile
     const bool one_pool = static_cast<const void*>(kpool) == static_cast<const void*>(vpool) && dk == dv;
-    float* Vs = one_pool ? Ks : Ks + KEYS * dkp;  // [KEYS][dvp]
+    // the queries are staged once and then live in registers, a lane's quarter of its row; the tiles of values take
+    // their place in LDS
+    float* Qs = lds;                              // [MROWS][dkp], later [KEYS][dvp]
+    float* Ks = lds + mfma_first_floats(dk, dv, one_pool);      // [KEYS][dkp]
+    float* Vs = one_pool ? Ks : lds;
     const int tile = blockIdx.x, g = blockIdx.y, chunk = blockIdx.z;
     const int seq = tiles[4 * tile], first_row = tiles[4 * tile + 1], n_tok = tiles[4 * tile + 2];
     const int first_pos = positions[first_row];
@@ -565,13 +576,18 @@ bias_attention_mfma_kernel(const T* __restrict__ qkv, int row_stride, const T* _
     const int wave_rows = std::min(16, n_rows - wave * 16);
     const int wave_last = wave_rows > 0 ? first_pos + (wave * 16 + wave_rows - 1) / heads_here : -1;
     float m = -INFINITY, l = 0.f;
-    floatx4_t acc[MAX_VCHUNKS * 4];               // dv / 16 blocks of [4 dims] of the lane's row
+    floatx4_t acc[DVB];                           // dv / 16 blocks of [4 dims] of the lane's row
 #pragma unroll
-    for (int db = 0; db < MAX_VCHUNKS * 4; ++db) acc[db] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+    for (int db = 0; db < DVB; ++db) acc[db] = floatx4_t{0.f, 0.f, 0.f, 0.f};
     const int dvb = dv / 16, qsteps = dk / 16;    // value blocks; 16-byte reads of a lane's quarter of a row
     const int last_pos = first_pos + n_tok - 1;
     const int32_t* table = block_table + static_cast<size_t>(seq) * table_width;
     const float* qrow = Qs + row * dkp + kg * (dk / 4);
+    __syncthreads();                              // the queries are all there
+    float4 qreg[QS];
+#pragma unroll
+    for (int t4 = 0; t4 < QS; ++t4)
+        qreg[t4] = t4 < qsteps ? *reinterpret_cast<const float4*>(qrow + 4 * t4) : make_float4(0.f, 0.f, 0.f, 0.f);
     const KeyWalk walk(first_pos, last_pos, window, keep_first);
     for (int v = 0; v < walk.steps; ++v) {
         const int k0 = walk.first_key(v);
@@ -584,15 +600,18 @@ bias_attention_mfma_kernel(const T* __restrict__ qkv, int row_stride, const T* _
         floatx4_t sc[KEYS / 16];
 #pragma unroll
         for (int j = 0; j < KEYS / 16; ++j) sc[j] = floatx4_t{0.f, 0.f, 0.f, 0.f};
-        for (int t4 = 0; t4 < qsteps; ++t4) {
-            const float4 qv = *reinterpret_cast<const float4*>(qrow + 4 * t4);
 #pragma unroll
-            for (int j = 0; j < KEYS / 16; ++j) {
-                const float4 kv = *reinterpret_cast<const float4*>(Ks + (16 * j + i) * dkp + kg * (dk / 4) + 4 * t4);
-                sc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(kv.x, qv.x, sc[j], 0, 0, 0);
-                sc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(kv.y, qv.y, sc[j], 0, 0, 0);
-                sc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(kv.z, qv.z, sc[j], 0, 0, 0);
-                sc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(kv.w, qv.w, sc[j], 0, 0, 0);
+        for (int t4 = 0; t4 < QS; ++t4) {
+            if (t4 < qsteps) {
+                const float4 qv = qreg[t4];
+#pragma unroll
+                for (int j = 0; j < KEYS / 16; ++j) {
+                    const float4 kv = *reinterpret_cast<const float4*>(Ks + (16 * j + i) * dkp + kg * (dk / 4) + 4 * t4);
+                    sc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(kv.x, qv.x, sc[j], 0, 0, 0);
+                    sc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(kv.y, qv.y, sc[j], 0, 0, 0);
+                    sc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(kv.z, qv.z, sc[j], 0, 0, 0);
+                    sc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(kv.w, qv.w, sc[j], 0, 0, 0);
+                }
             }
         }
         float top = -INFINITY;
@@ -625,7 +644,7 @@ bias_attention_mfma_kernel(const T* __restrict__ qkv, int row_stride, const T* _
         l = l * alpha + groups4(sum, false);
         m = m_new;
 #pragma unroll
-        for (int db = 0; db < MAX_VCHUNKS * 4; ++db) {
+        for (int db = 0; db < DVB; ++db) {
             if (db < dvb) {
                 floatx4_t a = acc[db] * alpha;
 #pragma unroll
@@ -645,7 +664,7 @@ bias_attention_mfma_kernel(const T* __restrict__ qkv, int row_stride, const T* _
         inv = out_scale * w / (l * w + expf(sk - M));
     }
 #pragma unroll
-    for (int db = 0; db < MAX_VCHUNKS * 4; ++db) {
+    for (int db = 0; db < DVB; ++db) {
         if (db < dvb) {
 #pragma unroll
             for (int r = 0; r < 4; ++r) st(orow + 16 * db + r, acc[db][r] * inv);
@@ -750,9 +769,9 @@ NI_EXPORT int ni_bias_attention(const void* qkv, int row_stride, const void* kpo
     return NI_LAUNCH_RESULT();
 }
 
-// staging memory of the matrix-core kernel: queries, a tile of keys and, unless they are the keys' pool, one of values
+// staging memory of the matrix-core kernel: the queries (then the tiles of values) and a tile of keys
 static size_t mfma_lds_bytes(int dk, int dv, bool one_pool) {
-    return (static_cast<size_t>(MROWS + KEYS) * (dk + 4) + (one_pool ? 0 : static_cast<size_t>(KEYS) * (dv + 4))) * sizeof(float);
+    return (mfma_first_floats(dk, dv, one_pool) + static_cast<size_t>(KEYS) * (dk + 4)) * sizeof(float);
 }
 
 // rows of (token, head) of a tile of the matrix-core kernel; 0 where it does not take these sizes.  `one_pool`: keys
@@ -760,6 +779,29 @@ static size_t mfma_lds_bytes(int dk, int dv, bool one_pool) {
 NI_EXPORT int ni_bias_attention_mfma_rows(int dk, int dv, int one_pool) {
     if (dk % 16 || dv % 16 || dk < 16 || dv < 16 || dv > MAX_VCHUNKS * WAVE || (one_pool && dk != dv)) return 0;
     return mfma_lds_bytes(dk, dv, one_pool != 0) <= 160 * 1024 ? MROWS : 0;
+}
+
+struct MfmaArgs {
+    const void *qkv; int row_stride; const void *kpool, *vpool, *block_table; int table_width; const void *tiles, *positions, *bias;
+    int distances; void* out; int H, G, dk, dv, page_size; float scale, temp_coef; int temp_every, heads_per_chunk;
+    bool k_pieces, v_pieces; int window, keep_first; float out_scale; const void* sink;
+};
+
+template <typename T, int QS, int DVB>
+static hipError_t launch_mfma(const MfmaArgs& a, dim3 grid, size_t lds, hipStream_t stream) {
+    static size_t allowed = 48 * 1024;            // of this instance of the kernel
+    if (lds > allowed) {
+        const hipError_t err = hipFuncSetAttribute((const void*)bias_attention_mfma_kernel<T, QS, DVB>,
+                                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (err != hipSuccess) return err;
+        allowed = lds;
+    }
+    bias_attention_mfma_kernel<T, QS, DVB><<<grid, WAVES * WAVE, lds, stream>>>(
+        (const T*)a.qkv, a.row_stride, (const T*)a.kpool, (const T*)a.vpool, (const int32_t*)a.block_table, a.table_width,
+        (const int32_t*)a.tiles, (const int32_t*)a.positions, (const float*)a.bias, a.distances, (T*)a.out, a.H, a.G, a.dk, a.dv,
+        a.page_size, a.scale, a.temp_coef, a.temp_every, a.heads_per_chunk, a.k_pieces, a.v_pieces, a.window, a.keep_first,
+        a.out_scale, (const float*)a.sink);
+    return hipSuccess;
 }
 
 // tiles of up to 64 rows (tokens * heads of a chunk), no runs: for steps with portions of prompts
@@ -778,25 +820,14 @@ NI_EXPORT int ni_bias_attention_mfma(const void* qkv, int row_stride, const void
     const bool k_pieces = dk % vec == 0 && reinterpret_cast<uintptr_t>(kpool) % 16 == 0;
     const bool v_pieces = dv % vec == 0 && reinterpret_cast<uintptr_t>(vpool) % 16 == 0;
     dim3 grid(n_tiles, G, (group + heads_per_chunk - 1) / heads_per_chunk);
-    hipError_t err = hipSuccess;
-    if (dtype == 0) {
-        static size_t allowed = 48 * 1024;
-        if (lds > allowed && (allowed = lds))
-            err = hipFuncSetAttribute((const void*)bias_attention_mfma_kernel<float>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (err != hipSuccess) return (int)err;
-        bias_attention_mfma_kernel<float><<<grid, WAVES * WAVE, lds, stream>>>(
-            (const float*)qkv, row_stride, (const float*)kpool, (const float*)vpool, (const int32_t*)block_table, table_width,
-            (const int32_t*)tiles, (const int32_t*)positions, (const float*)bias, distances, (float*)out, H, G, dk, dv, page_size,
-            scale, temp_coef, temp_every, heads_per_chunk, k_pieces, v_pieces, window, keep_first, out_scale, (const float*)sink);
-    } else {
-        static size_t allowed = 48 * 1024;
-        if (lds > allowed && (allowed = lds))
-            err = hipFuncSetAttribute((const void*)bias_attention_mfma_kernel<bf16_t>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (err != hipSuccess) return (int)err;
-        bias_attention_mfma_kernel<bf16_t><<<grid, WAVES * WAVE, lds, stream>>>(
-            (const bf16_t*)qkv, row_stride, (const bf16_t*)kpool, (const bf16_t*)vpool, (const int32_t*)block_table, table_width,
-            (const int32_t*)tiles, (const int32_t*)positions, (const float*)bias, distances, (bf16_t*)out, H, G, dk, dv, page_size,
-            scale, temp_coef, temp_every, heads_per_chunk, k_pieces, v_pieces, window, keep_first, out_scale, (const float*)sink);
-    }
+    const MfmaArgs args{qkv, row_stride, kpool, vpool, block_table, table_width, tiles, positions, bias, distances, out, H, G, dk, dv,
+                        page_size, scale, temp_coef, temp_every, heads_per_chunk, k_pieces, v_pieces, window, keep_first, out_scale, sink};
+    hipError_t err;
+    // the smallest arrays of registers that hold these sizes
+    if (dk <= 64 && dv <= 64) err = dtype == 0 ? launch_mfma<float, 4, 4>(args, grid, lds, stream) : launch_mfma<bf16_t, 4, 4>(args, grid, lds, stream);
+    else if (dk <= 128 && dv <= 64) err = dtype == 0 ? launch_mfma<float, 8, 4>(args, grid, lds, stream) : launch_mfma<bf16_t, 8, 4>(args, grid, lds, stream);
+    else if (dk <= 128) err = dtype == 0 ? launch_mfma<float, 8, 16>(args, grid, lds, stream) : launch_mfma<bf16_t, 8, 16>(args, grid, lds, stream);
+    else err = dtype == 0 ? launch_mfma<float, 16, 16>(args, grid, lds, stream) : launch_mfma<bf16_t, 16, 16>(args, grid, lds, stream);
+    if (err != hipSuccess) return (int)err;
     return NI_LAUNCH_RESULT();
 }
